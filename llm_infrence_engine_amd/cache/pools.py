@@ -49,7 +49,7 @@ class CachePools:
         self.state: Dict[int, tuple] = {}
         for run, need in layout.state_needs.items():
             needs = need if isinstance(need, tuple) else (need,)
-            self.state[run] = tuple(torch.zeros((max_requests + 1, *n.shape), dtype=n.dtype, device=rt.device) for n in needs)
+            self.state[run] = tuple(torch.zeros((max_requests + 1, *n.shape), dtype=n.dtype or rt.dtype, device=rt.device) for n in needs)
 
     def total_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for g in self.pages for t in g.values()) + \

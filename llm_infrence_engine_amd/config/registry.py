@@ -1,6 +1,7 @@
 """One registry from an architecture's name to its typed configuration (and through it, its model).
 
-``config.json`` names the architecture in ``architectures[0]`` (``model_type`` is the fallback).
+``config.json`` names the architecture in ``architectures[0]`` or in ``architecture`` (``model_type`` is the
+fallback).
 The reference has no registry: its loader builds the one model it knows
 (src/miniserve/loader.py:38-39) and never reads ``architectures``.
 """
@@ -46,6 +47,8 @@ def config_from_dict(d: dict):
     archs = d.get("architectures")
     if archs:
         name = archs[0]
+    elif isinstance(d.get("architecture"), str):
+        name = d["architecture"]
     elif d.get("model_type") in _MODEL_TYPES:
         name = _MODEL_TYPES[d["model_type"]]
     elif len(_ARCHITECTURES) == 1:

@@ -80,6 +80,7 @@ class ModelSpec:
     order: Tuple[Run, ...]
     final_norm: PartSpec
     head: PartSpec
+    ignorable: Tuple[str, ...] = ()    # tensors a checkpoint may hold that no part of this model reads
 
     def __post_init__(self):
         for i, run in enumerate(self.order):

@@ -145,4 +145,47 @@ int ms_sample(const float* logits, long long ld, int n_rows, int vocab, const fl
               const float* top_p, const unsigned long long* seeds, const int* draw_index, int* out, void* workspace,
               int use_top_k, int use_top_p, hipStream_t stream);
 
+// ---- mixers with a fixed-size state (csrc/sequence.hip).  A step's requests: tokens q_start[r]..q_start[r+1]-1, state
+// slot state_slots[r]; token_req [n_tokens]; n_live_tokens (may be null): tokens from there on belong to no request.
+// Short causal convolution per channel: w float [channels, taps] (last column: the current token), state
+// [slots, taps - 1, channels] in `dtype`.  mode 0: the sum, 1: x + the sum, 2: silu(the sum).  out must not be x.
+// With update_state the state becomes the last taps - 1 inputs of every request that has tokens.
+int ms_short_conv(const void* x, long long x_stride, const float* w, void* state, const int* token_req,
+                  const int* q_start, const int* state_slots, const int* n_live_tokens, void* out, long long out_stride,
+                  int n_tokens, int n_requests, int channels, int taps, int mode, int update_state, int dtype,
+                  hipStream_t stream);
+
+// Gated delta rule with a decay per head and key channel.  q, k [n, kv_heads * dim], v [n, heads * vdim], b [n, heads]
+// in `dtype` (rows qkv_stride / b_stride apart); a float [n, heads * dim] (the decay's input before dt_bias);
+// state float [slots, heads, dim, vdim]; out float [n, heads * vdim].
+int ms_gated_delta(const void* q, const void* k, const void* v, long long qkv_stride, const float* a, const void* b,
+                   long long b_stride, const float* A_log, const float* dt_bias, float* state, const int* q_start,
+                   const int* state_slots, float* out, int n_requests, int heads, int kv_heads, int dim, int vdim,
+                   int dtype, hipStream_t stream);
+
+// out[n, h, :] = o[n, h, :] / rms(o[n, h, :]) * weight * sigmoid(gate[n, h, :]); o float, gate and out in `dtype`.
+int ms_gated_head_norm(const float* o, const float* weight, const void* gate, long long gate_stride, void* out,
+                       int n_tokens, int heads, int vdim, float eps, int dtype, hipStream_t stream);
+
+// xIELU with pq = (p, q) on the device.
+int ms_xielu(const void* x, const float* pq, void* out, long long total, int dtype, hipStream_t stream);
+
+// ---- attention through a latent (csrc/latent_attention.hip); strides in elements
+int ms_head_matmul(const void* in, long long in_tok, long long in_head, const void* M, void* out, long long out_tok,
+                   long long out_head, const void* gate, long long gate_tok, int n_tokens, int heads, int I, int J,
+                   int dtype, int out_dtype, hipStream_t stream);
+int ms_rms_norm_rows(const void* in, long long in_stride, const float* weight, void* out, long long out_stride, int n_rows,
+                     int width, float eps, int dtype, hipStream_t stream);
+int ms_rotary_pairs(const void* src, long long src_tok, long long src_head, void* dst, long long dst_tok,
+                    long long dst_head, const int* positions, const float* inv_freq, int n_tokens, int heads, int width,
+                    int dims, int dtype, hipStream_t stream);
+int ms_latent_kv_store(const void* kv, long long kv_stride, const float* norm_w, float eps, const int* positions,
+                       const float* inv_freq, const int* slots, void* c_pages, void* r_pages, int n_tokens, int C, int R,
+                       int dims, int dtype, hipStream_t stream);
+int ms_latent_attention(const void* q, long long q_tok, long long q_head, const void* c_pages, const void* r_pages,
+                        const int* block_table, int table_stride, const int* table_rows, const int* n_live_tokens,
+                        const int* token_req, const int* positions, const float* sink, void* out, long long out_tok,
+                        long long out_head, int n_tokens, int heads, int C, int R, int page_size, long long num_pages,
+                        float scale, int window, int dtype, hipStream_t stream);
+
 }  // extern "C"

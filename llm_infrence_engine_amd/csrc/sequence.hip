@@ -1,0 +1,309 @@
+// Kernels of mixers that carry a fixed-size state from token to token instead of reading a cache of keys:
+// a short causal convolution over time per channel (with the last taps - 1 inputs as state), the gated delta
+// rule with one decay per head and key channel, and the gated RMS norm of its read-out.
+// A step is a ragged batch: request r owns the tokens q_start[r] .. q_start[r+1]-1 (a portion of a prompt or
+// one decoded token) and the state slot state_slots[r]; requests without tokens and tokens of no request pad a
+// captured batch and are left alone.  All recurrences, decays, gates and norms are float in every mode.
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+constexpr int MAX_TAPS = 8;
+
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// ------------------------------------------------------------------------------------------------
+// y[n, c] = act(sum_j w[c, j] * in(t - taps + 1 + j)) (+ x[n, c]), t the token's index within its portion;
+// in(i) is the portion's own input for i >= 0 and the state (the taps - 1 inputs before the portion) for i < 0.
+// mode 0: the sum; 1: x + the sum; 2: silu of the sum.
+template <typename T>
+__global__ void short_conv_kernel(const T* __restrict__ x, size_t x_stride, const float* __restrict__ w,
+                                  const T* __restrict__ state, const int* __restrict__ token_req,
+                                  const int* __restrict__ q_start, const int* __restrict__ state_slots,
+                                  const int* __restrict__ n_live_tokens, T* __restrict__ out, size_t out_stride,
+                                  int C, int taps, int mode) {
+  const int n = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  if (n_live_tokens && n >= *n_live_tokens) return;
+  const int r = token_req[n];
+  const int s = q_start[r];
+  const int t = n - s;
+  const T* st = state + (size_t)state_slots[r] * (taps - 1) * C;
+  float acc = 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int i = t - taps + 1 + j;
+    const float v = i >= 0 ? to_float(x[(size_t)(s + i) * x_stride + c]) : to_float(st[(size_t)(taps - 1 + i) * C + c]);
+    acc = fmaf(w[(size_t)c * taps + j], v, acc);
+  }
+  if (mode == 1) acc += to_float(x[(size_t)n * x_stride + c]);
+  else if (mode == 2) acc = acc * sigmoid_f(acc);
+  out[(size_t)n * out_stride + c] = from_float<T>(acc);
+}
+
+// After the convolution: the state of every request with tokens becomes its last taps - 1 inputs.
+template <typename T>
+__global__ void short_conv_update_kernel(const T* __restrict__ x, size_t x_stride, T* __restrict__ state,
+                                         const int* __restrict__ q_start, const int* __restrict__ state_slots,
+                                         int C, int taps) {
+  const int r = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int s = q_start[r], L = q_start[r + 1] - s;
+  if (L <= 0) return;
+  T* st = state + (size_t)state_slots[r] * (taps - 1) * C;
+  T keep[MAX_TAPS];
+  const int hist = taps - 1;
+#pragma unroll
+  for (int i = 0; i < MAX_TAPS - 1; ++i)
+    if (i < hist) {
+      const int src = L - hist + i;   // index within the portion; negative: still in the old state
+      keep[i] = src >= 0 ? x[(size_t)(s + src) * x_stride + c] : st[(size_t)(src + hist) * C + c];
+    }
+#pragma unroll
+  for (int i = 0; i < MAX_TAPS - 1; ++i)
+    if (i < hist) st[(size_t)i * C + c] = keep[i];
+}
+
+// ------------------------------------------------------------------------------------------------
+// The gated delta rule.  Per request and head, S [D, E] float, token by token:
+//   S <- g * S (row i by g_i);  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+// with q, k made unit vectors per head (q also times D^-1/2), beta = sigmoid(b) and
+// g = exp(-exp(A_log_h) * softplus(a + dt_bias)).  Column j of S depends on no other column, so a column is
+// held in the registers of LPC neighbouring lanes (DPT rows each) for the whole portion.  Tokens are staged a
+// chunk at a time: the chunk's q, k (normalised), g, beta and v are worked out by all threads in parallel into
+// LDS, then the chunk's tokens are walked in order.
+constexpr int DELTA_CHUNK = 16;
+
+template <typename T, int DPT>
+__global__ void __launch_bounds__(256)
+gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, size_t qkv_stride,
+                   const float* __restrict__ a, const T* __restrict__ b, size_t b_stride,
+                   const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ state,
+                   const int* __restrict__ q_start, const int* __restrict__ state_slots, float* __restrict__ out,
+                   int H, int G, int D, int E, int lpc, int cols_per_block) {
+  extern __shared__ __align__(16) float lds[];
+  const int Dp = DPT * lpc;                       // padded key size
+  float* qs = lds;                                // [CHUNK][Dp]
+  float* ks = qs + DELTA_CHUNK * Dp;
+  float* gs = ks + DELTA_CHUNK * Dp;
+  float* vs = gs + DELTA_CHUNK * Dp;              // [CHUNK][cols_per_block]
+  float* bs = vs + DELTA_CHUNK * cols_per_block;  // [CHUNK]
+  const int r = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * cols_per_block;
+  const int kvh = h / (H / G);
+  const int s0 = q_start[r], L = q_start[r + 1] - s0;
+  if (L <= 0) return;
+  const int tid = threadIdx.x, lane = tid & (MS_WAVE - 1), wave = tid / MS_WAVE, nwaves = blockDim.x / MS_WAVE;
+  const int part = tid % lpc, col = col0 + tid / lpc;
+  const bool live = col < E && tid / lpc < cols_per_block;
+  float* Sg = state + (((size_t)state_slots[r] * H + h) * D) * E;
+  float S[DPT];
+#pragma unroll
+  for (int ii = 0; ii < DPT; ++ii) {
+    const int i = part * DPT + ii;
+    S[ii] = (live && i < D) ? Sg[(size_t)i * E + col] : 0.f;
+  }
+  const float rate = expf(A_log[h]);
+  const float q_scale = 1.0f / sqrtf((float)D);
+
+  for (int c0 = 0; c0 < L; c0 += DELTA_CHUNK) {
+    const int cn = min(DELTA_CHUNK, L - c0);
+    __syncthreads();   // the chunk before is done with the staging area
+    for (int t = wave; t < cn; t += nwaves) {        // a wave normalises a token's q and k
+      const size_t n = (size_t)(s0 + c0 + t);
+      const T* qp = q + n * qkv_stride + (size_t)kvh * D;
+      const T* kp = k + n * qkv_stride + (size_t)kvh * D;
+      float sq = 0.f, sk = 0.f;
+      for (int i = lane; i < D; i += MS_WAVE) {
+        const float a0 = to_float(qp[i]), a1 = to_float(kp[i]);
+        sq = fmaf(a0, a0, sq);
+        sk = fmaf(a1, a1, sk);
+      }
+      sq = wave_sum(sq);
+      sk = wave_sum(sk);
+      const float iq = q_scale / sqrtf(sq + 1e-6f), ik = 1.0f / sqrtf(sk + 1e-6f);
+      const float* ap = a + n * (size_t)H * D + (size_t)h * D;
+      for (int i = lane; i < Dp; i += MS_WAVE) {
+        const bool in = i < D;
+        qs[t * Dp + i] = in ? to_float(qp[i]) * iq : 0.f;
+        ks[t * Dp + i] = in ? to_float(kp[i]) * ik : 0.f;
+        gs[t * Dp + i] = in ? expf(-rate * softplus_f(ap[i] + dt_bias[(size_t)h * D + i])) : 1.f;
+      }
+      if (lane == 0) bs[t] = sigmoid_f(to_float(b[n * b_stride + h]));
+    }
+    for (int e = tid; e < cn * cols_per_block; e += blockDim.x) {
+      const int t = e / cols_per_block, j = e - t * cols_per_block;
+      vs[e] = col0 + j < E ? to_float(v[(size_t)(s0 + c0 + t) * qkv_stride + (size_t)h * E + col0 + j]) : 0.f;
+    }
+    __syncthreads();
+    for (int t = 0; t < cn; ++t) {
+      const float* qt = qs + t * Dp + part * DPT;
+      const float* kt = ks + t * Dp + part * DPT;
+      const float* gt = gs + t * Dp + part * DPT;
+      float kv = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < DPT; ii += 4) {
+        const float4 g4 = *reinterpret_cast<const float4*>(gt + ii);
+        const float4 k4 = *reinterpret_cast<const float4*>(kt + ii);
+        S[ii] *= g4.x; S[ii + 1] *= g4.y; S[ii + 2] *= g4.z; S[ii + 3] *= g4.w;
+        kv = fmaf(S[ii], k4.x, kv); kv = fmaf(S[ii + 1], k4.y, kv);
+        kv = fmaf(S[ii + 2], k4.z, kv); kv = fmaf(S[ii + 3], k4.w, kv);
+      }
+      for (int o = 1; o < lpc; o <<= 1) kv += __shfl_xor(kv, o, MS_WAVE);
+      const float u = bs[t] * (vs[t * cols_per_block + tid / lpc] - kv);
+      float o_sum = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < DPT; ii += 4) {
+        const float4 k4 = *reinterpret_cast<const float4*>(kt + ii);
+        const float4 q4 = *reinterpret_cast<const float4*>(qt + ii);
+        S[ii] = fmaf(k4.x, u, S[ii]); S[ii + 1] = fmaf(k4.y, u, S[ii + 1]);
+        S[ii + 2] = fmaf(k4.z, u, S[ii + 2]); S[ii + 3] = fmaf(k4.w, u, S[ii + 3]);
+        o_sum = fmaf(S[ii], q4.x, o_sum); o_sum = fmaf(S[ii + 1], q4.y, o_sum);
+        o_sum = fmaf(S[ii + 2], q4.z, o_sum); o_sum = fmaf(S[ii + 3], q4.w, o_sum);
+      }
+      for (int o = 1; o < lpc; o <<= 1) o_sum += __shfl_xor(o_sum, o, MS_WAVE);
+      if (live && part == 0) out[((size_t)(s0 + c0 + t) * H + h) * E + col] = o_sum;
+    }
+  }
+#pragma unroll
+  for (int ii = 0; ii < DPT; ++ii) {
+    const int i = part * DPT + ii;
+    if (live && i < D) Sg[(size_t)i * E + col] = S[ii];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// y[n, h, :] = o[n, h, :] / sqrt(mean(o[n, h, :]^2) + eps) * w[:] * sigmoid(gate[n, h, :]); one wave per (token, head).
+template <typename T>
+__global__ void gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ w,
+                                       const T* __restrict__ gate, size_t gate_stride, T* __restrict__ out,
+                                       long long items, int H, int E, float eps) {
+  const int lane = threadIdx.x & (MS_WAVE - 1);
+  const long long item = (long long)blockIdx.x * (blockDim.x / MS_WAVE) + threadIdx.x / MS_WAVE;
+  if (item >= items) return;
+  const long long n = item / H;
+  const int h = (int)(item - n * H);
+  const float* op = o + (size_t)item * E;
+  float ss = 0.f;
+  for (int i = lane; i < E; i += MS_WAVE) ss = fmaf(op[i], op[i], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)E + eps);
+  const T* gp = gate + (size_t)n * gate_stride + (size_t)h * E;
+  T* yp = out + (size_t)item * E;
+  for (int i = lane; i < E; i += MS_WAVE)
+    yp[i] = from_float<T>(op[i] * inv * w[i] * sigmoid_f(to_float(gp[i])));
+}
+
+// ------------------------------------------------------------------------------------------------
+// The xIELU activation with its two learned numbers (p, q):  z > 0: softplus(p) z^2 + z/2;
+// z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2.
+template <typename T>
+__global__ void xielu_kernel(const T* __restrict__ x, const float* __restrict__ pq, T* __restrict__ out, size_t total) {
+  const float ap = softplus_f(pq[0]), an = 0.5f + softplus_f(pq[1]);
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += stride) {
+    const float z = to_float(x[i]);
+    const float y = z > 0.f ? fmaf(ap * z, z, 0.5f * z) : fmaf(an, expm1f(z) - z, 0.5f * z);
+    out[i] = from_float<T>(y);
+  }
+}
+
+}  // namespace
+
+extern "C" int ms_short_conv(const void* x, long long x_stride, const float* w, void* state, const int* token_req,
+                             const int* q_start, const int* state_slots, const int* n_live_tokens, void* out,
+                             long long out_stride, int n_tokens, int n_requests, int channels, int taps, int mode,
+                             int update_state, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return MS_OK;
+  if (channels <= 0 || taps < 1 || mode < 0 || mode > 2 || n_requests <= 0) return MS_BAD_ARG;
+  if (taps > MAX_TAPS) return MS_UNSUPPORTED;
+  const int threads = channels >= 256 ? 256 : 64;
+  const int cblocks = (channels + threads - 1) / threads;
+  if (cblocks > 65535 || n_requests > 65535) return MS_UNSUPPORTED;
+  dim3 block(threads), grid(n_tokens, cblocks), ugrid(cblocks, n_requests);
+#define LAUNCH(T)                                                                                                       \
+  do {                                                                                                                  \
+    short_conv_kernel<T><<<grid, block, 0, stream>>>((const T*)x, (size_t)x_stride, w, (const T*)state, token_req,     \
+                                                     q_start, state_slots, n_live_tokens, (T*)out, (size_t)out_stride, \
+                                                     channels, taps, mode);                                             \
+    if (update_state && taps > 1)                                                                                       \
+      short_conv_update_kernel<T><<<ugrid, block, 0, stream>>>((const T*)x, (size_t)x_stride, (T*)state, q_start,      \
+                                                               state_slots, channels, taps);                            \
+  } while (0)
+  if (dtype == MS_F32) LAUNCH(float);
+  else if (dtype == MS_BF16) LAUNCH(bf16);
+  else return MS_BAD_ARG;
+#undef LAUNCH
+  return ms_launch_status();
+}
+
+extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long long qkv_stride, const float* a,
+                              const void* b, long long b_stride, const float* A_log, const float* dt_bias,
+                              float* state, const int* q_start, const int* state_slots, float* out, int n_requests,
+                              int heads, int kv_heads, int dim, int vdim, int dtype, hipStream_t stream) {
+  if (n_requests <= 0) return MS_OK;
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return MS_BAD_ARG;
+  if (dim > 512 || n_requests > 65535 || heads > 65535) return MS_UNSUPPORTED;
+  // rows of a column a lane holds (DPT) and lanes a column is spread over (lpc): as few lanes as keep DPT <= 64
+  int lpc = 1;
+  while ((dim + lpc - 1) / lpc > 64) lpc *= 2;
+  // a short column leaves registers free: spread it further while the block still has a wave's worth of columns
+  while (lpc < 8 && (dim + lpc - 1) / lpc > 16 && vdim * lpc < 128) lpc *= 2;
+  const int per = (dim + lpc - 1) / lpc;
+  const int dpt = per <= 8 ? 8 : per <= 16 ? 16 : per <= 32 ? 32 : 64;
+  int threads = vdim * lpc;
+  threads = threads >= 256 ? 256 : ((threads + MS_WAVE - 1) / MS_WAVE) * MS_WAVE;
+  const int cols = threads / lpc;
+  dim3 grid((vdim + cols - 1) / cols, heads, n_requests), block(threads);
+  const size_t lds = (size_t)DELTA_CHUNK * (3 * (size_t)dpt * lpc + cols + 1) * sizeof(float);
+  if (lds > 65536) return MS_UNSUPPORTED;
+#define LAUNCH(T, DPT)                                                                                                  \
+  gated_delta_kernel<T, DPT><<<grid, block, lds, stream>>>((const T*)q, (const T*)k, (const T*)v, (size_t)qkv_stride, \
+                                                           a, (const T*)b, (size_t)b_stride, A_log, dt_bias, state,   \
+                                                           q_start, state_slots, out, heads, kv_heads, dim, vdim,     \
+                                                           lpc, cols)
+#define BY_DPT(T)                                                                                                       \
+  do {                                                                                                                  \
+    if (dpt == 8) LAUNCH(T, 8);                                                                                         \
+    else if (dpt == 16) LAUNCH(T, 16);                                                                                  \
+    else if (dpt == 32) LAUNCH(T, 32);                                                                                  \
+    else LAUNCH(T, 64);                                                                                                 \
+  } while (0)
+  if (dtype == MS_F32) BY_DPT(float);
+  else if (dtype == MS_BF16) BY_DPT(bf16);
+  else return MS_BAD_ARG;
+#undef BY_DPT
+#undef LAUNCH
+  return ms_launch_status();
+}
+
+extern "C" int ms_gated_head_norm(const float* o, const float* weight, const void* gate, long long gate_stride,
+                                  void* out, int n_tokens, int heads, int vdim, float eps, int dtype,
+                                  hipStream_t stream) {
+  if (n_tokens <= 0) return MS_OK;
+  if (heads <= 0 || vdim <= 0) return MS_BAD_ARG;
+  const long long items = (long long)n_tokens * heads;
+  const int waves = 4;
+  dim3 grid((unsigned)((items + waves - 1) / waves)), block(waves * MS_WAVE);
+  if (dtype == MS_F32)
+    gated_head_norm_kernel<float><<<grid, block, 0, stream>>>(o, weight, (const float*)gate, (size_t)gate_stride,
+                                                              (float*)out, items, heads, vdim, eps);
+  else if (dtype == MS_BF16)
+    gated_head_norm_kernel<bf16><<<grid, block, 0, stream>>>(o, weight, (const bf16*)gate, (size_t)gate_stride,
+                                                             (bf16*)out, items, heads, vdim, eps);
+  else return MS_BAD_ARG;
+  return ms_launch_status();
+}
+
+extern "C" int ms_xielu(const void* x, const float* pq, void* out, long long total, int dtype, hipStream_t stream) {
+  if (total <= 0) return MS_OK;
+  int blocks = (int)((total + 255) / 256);
+  if (blocks > 8192) blocks = 8192;
+  if (dtype == MS_F32) xielu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)x, pq, (float*)out, (size_t)total);
+  else if (dtype == MS_BF16) xielu_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)x, pq, (bf16*)out, (size_t)total);
+  else return MS_BAD_ARG;
+  return ms_launch_status();
+}

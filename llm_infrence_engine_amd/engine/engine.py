@@ -36,7 +36,7 @@ def memory_beside_the_pages(config: EngineConfig, model: Model, layout: CacheLay
             size = 1
             for s in n.shape:
                 size *= s
-            total += (config.max_seqs + 1) * size * torch.empty(0, dtype=n.dtype).element_size()
+            total += (config.max_seqs + 1) * size * (n.dtype or model.rt.dtype).itemsize
     total += len(layout.group_keys) * (config.max_seqs + 1) * config.pages_per_request * 4
     widest = max([model.spec.hidden_size * 4] + [s.shape[0] * itemsize for s in model.tensor_specs()
                                                   if s.role == "matrix" and len(s.shape) == 2

@@ -72,6 +72,22 @@ _SIGNATURES = {
     "ms_sample": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                   _c_ptr],
     "ms_sample_workspace_bytes": [_c_int],
+    "ms_short_conv": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int,
+                      _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_gated_delta": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_gated_head_norm": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "ms_xielu": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
+    "ms_head_matmul": [_c_ptr, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_ll, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int,
+                       _c_int, _c_int, _c_ptr],
+    "ms_rms_norm_rows": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "ms_rotary_pairs": [_c_ptr, _c_ll, _c_ll, _c_ptr, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
+                        _c_ptr],
+    "ms_latent_kv_store": [_c_ptr, _c_ll, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+                           _c_int, _c_int, _c_ptr],
+    "ms_latent_attention": [_c_ptr, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                            _c_ptr, _c_ll, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float, _c_int, _c_int,
+                            _c_ptr],
 }
 
 _fn = {}
@@ -819,3 +835,203 @@ def paged_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, num_heads: int,
                                     num_heads, scale, ctx.max_q_len, ctx.max_context_len, window, kv.table_rows)
     return paged_attention_generic(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.token_req, ctx.positions, out,
                                    num_heads, scale, window, kv.v_transposed, kv.table_rows, ctx.n_live_tokens)
+
+
+# ------------------------------------------------------------------------------------------------ state-carrying mixers
+CONV_SUM, CONV_ADD_INPUT, CONV_SILU = 0, 1, 2
+MAX_CONV_TAPS = 8
+
+
+def _rows2d(t: torch.Tensor, name: str, dtype=None, cols=None):
+    """A matrix whose rows may be slices of wider rows (unit stride along a row)."""
+    _check(t, name, dtype, contiguous=False)
+    if t.dim() != 2 or t.stride(1) != 1 or (cols is not None and t.shape[1] != cols):
+        raise ValueError(f"{name} must be [rows, {cols if cols is not None else 'columns'}] with unit stride along rows, "
+                         f"got {list(t.shape)} strides {t.stride()}")
+    return t.stride(0) if t.shape[0] > 1 else t.shape[1]
+
+
+def short_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx, out: torch.Tensor,
+               mode: int = CONV_SUM, update_state: bool = True) -> torch.Tensor:
+    """A causal convolution over time on every channel of ``x`` [N, C], for the step ``ctx`` describes:
+    out[n] = act(sum_j weight[:, j] * input(t - taps + 1 + j)), the last column meeting the token itself, inputs before a
+    request's portion taken from ``state`` [slots, taps - 1, C] (the request's slot; zero at a request's start).
+    ``mode``: CONV_SUM, CONV_ADD_INPUT (x + the sum) or CONV_SILU.  With ``update_state`` the state then becomes the
+    last taps - 1 inputs of every request of the step.  ``weight`` float [C, taps]."""
+    N, C = x.shape
+    xs = _rows2d(x, "x")
+    os_ = _rows2d(out, "out", x.dtype, C)
+    if out.shape[0] != N or out.data_ptr() == x.data_ptr():
+        raise ValueError("out must be another tensor of x's shape")
+    _check(weight, "weight", torch.float32, (C, None))
+    taps = weight.shape[1]
+    if taps > MAX_CONV_TAPS:
+        raise UnsupportedShape(f"the short convolution takes up to {MAX_CONV_TAPS} taps, got {taps}")
+    _check(state, "state", x.dtype, (None, max(1, taps - 1), C))
+    R = ctx.num_requests
+    _check(ctx.token_req, "token_req", torch.int32, (N,))
+    _check(ctx.q_start, "q_start", torch.int32, (R + 1,))
+    _check(ctx.state_slots, "state_slots", torch.int32, (R,))
+    _call("ms_short_conv", x.data_ptr(), xs, weight.data_ptr(), state.data_ptr(), ctx.token_req.data_ptr(),
+          ctx.q_start.data_ptr(), ctx.state_slots.data_ptr(), _ptr(ctx.n_live_tokens), out.data_ptr(), os_, N, R, C, taps,
+          mode, int(update_state), _code(x.dtype), _stream())
+    return out
+
+
+def gated_delta(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor,
+                dt_bias: torch.Tensor, state: torch.Tensor, ctx, out: torch.Tensor, heads: int, kv_heads: int, dim: int,
+                vdim: int) -> torch.Tensor:
+    """The gated delta rule over the step's portions, from and into ``state`` float [slots, heads, dim, vdim]:
+    per head and token  S <- g * S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q  with q, k made unit vectors
+    (q also times dim^-1/2), beta = sigmoid(b), g = exp(-exp(A_log) * softplus(a + dt_bias)).  q, k [N, kv_heads * dim],
+    v [N, heads * vdim] and b [N, heads] are row slices with one row stride for q, k, v; a float [N, heads * dim];
+    out float [N, heads * vdim]."""
+    N = q.shape[0]
+    sq = _rows2d(q, "q", None, kv_heads * dim)
+    sk = _rows2d(k, "k", q.dtype, kv_heads * dim)
+    sv = _rows2d(v, "v", q.dtype, heads * vdim)
+    if not (sq == sk == sv) and N > 1:
+        raise ValueError("q, k and v must be slices of rows of one width")
+    sb = _rows2d(b, "b", q.dtype, heads)
+    _check(a, "a", torch.float32, (N, heads * dim))
+    _check(A_log, "A_log", torch.float32, (heads,))
+    _check(dt_bias, "dt_bias", torch.float32, (heads * dim,))
+    _check(state, "state", torch.float32, (None, heads, dim, vdim))
+    _check(out, "out", torch.float32, (N, heads * vdim))
+    R = ctx.num_requests
+    _check(ctx.q_start, "q_start", torch.int32, (R + 1,))
+    _check(ctx.state_slots, "state_slots", torch.int32, (R,))
+    if heads % kv_heads:
+        raise ValueError(f"{heads} heads cannot share {kv_heads} query/key heads")
+    _call("ms_gated_delta", q.data_ptr(), k.data_ptr(), v.data_ptr(), sq, a.data_ptr(), b.data_ptr(), sb, A_log.data_ptr(),
+          dt_bias.data_ptr(), state.data_ptr(), ctx.q_start.data_ptr(), ctx.state_slots.data_ptr(), out.data_ptr(), R,
+          heads, kv_heads, dim, vdim, _code(q.dtype), _stream())
+    return out
+
+
+def gated_head_norm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, out: torch.Tensor, heads: int, vdim: int,
+                    eps: float) -> torch.Tensor:
+    """out[n, h] = o[n, h] / sqrt(mean(o[n, h]^2) + eps) * weight * sigmoid(gate[n, h]); o float [N, heads * vdim]."""
+    N = o.shape[0]
+    _check(o, "o", torch.float32, (N, heads * vdim))
+    _check(weight, "weight", torch.float32, (vdim,))
+    gs = _rows2d(gate, "gate", out.dtype, heads * vdim)
+    _check(out, "out", None, (N, heads * vdim))
+    _call("ms_gated_head_norm", o.data_ptr(), weight.data_ptr(), gate.data_ptr(), gs, out.data_ptr(), N, heads, vdim,
+          float(eps), _code(out.dtype), _stream())
+    return out
+
+
+def xielu(x: torch.Tensor, pq: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2, with pq = (p, q) float [2]."""
+    _check(x, "x")
+    _check(pq, "pq", torch.float32, (2,))
+    _check(out, "out", x.dtype, tuple(x.shape))
+    _call("ms_xielu", x.data_ptr(), pq.data_ptr(), out.data_ptr(), x.numel(), _code(x.dtype), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ attention through a latent
+def _heads3d(t: torch.Tensor, name: str, dtype=None):
+    _check(t, name, dtype, contiguous=False)
+    if t.dim() != 3 or t.stride(2) != 1:
+        raise ValueError(f"{name} must be [tokens, heads, width] with unit stride along the width, got {list(t.shape)} "
+                         f"strides {t.stride()}")
+    return t.stride(0), t.stride(1)
+
+
+def head_matmul(x: torch.Tensor, m: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[n, h, :] = x[n, h, :] @ m[h] (* sigmoid(gate[n, h, :])).  x [N, H, I] and out [N, H, J] may be views with any
+    token and head strides; m [H, I, J] contiguous; gate [N, H * J] rows."""
+    N, H, I = x.shape
+    xt, xh = _heads3d(x, "x")
+    _check(m, "m", x.dtype, (H, I, None))
+    J = m.shape[2]
+    ot, oh = _heads3d(out, "out")
+    if tuple(out.shape) != (N, H, J):
+        raise ValueError(f"out must be {[N, H, J]}, got {list(out.shape)}")
+    gs = 0
+    if gate is not None:
+        gs = _rows2d(gate, "gate", x.dtype, H * J)
+    _call("ms_head_matmul", x.data_ptr(), xt, xh, m.data_ptr(), out.data_ptr(), ot, oh, _ptr(gate), gs, N, H, I, J,
+          _code(x.dtype), _code(out.dtype), _stream())
+    return out
+
+
+def rms_norm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> torch.Tensor:
+    """out[n] = x[n] / sqrt(mean(x[n]^2) + eps) * weight for rows of an activation (row slices are fine)."""
+    N, C = x.shape
+    xs = _rows2d(x, "x")
+    os_ = _rows2d(out, "out", x.dtype, C)
+    _check(weight, "weight", torch.float32, (C,))
+    _call("ms_rms_norm_rows", x.data_ptr(), xs, weight.data_ptr(), out.data_ptr(), os_, N, C, float(eps), _code(x.dtype),
+          _stream())
+    return out
+
+
+def rotary_pairs(src: torch.Tensor, dst: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """dst[n, h] = src[n, h] with its first 2 * len(inv_freq) entries turned, entry 2i with entry 2i + 1, by
+    float(positions[n]) * inv_freq[i]; the rest is copied.  src, dst [N, H, width] views (dst may be src)."""
+    N, H, width = src.shape
+    st, sh = _heads3d(src, "src")
+    dt, dh = _heads3d(dst, "dst", src.dtype)
+    if tuple(dst.shape) != (N, H, width):
+        raise ValueError("dst must have src's shape")
+    _check(positions, "positions", torch.int32, (N,))
+    _check(inv_freq, "inv_freq", torch.float32)
+    dims = 2 * inv_freq.numel()
+    if dims > width:
+        raise ValueError(f"{dims} rotated entries do not fit a width of {width}")
+    _call("ms_rotary_pairs", src.data_ptr(), st, sh, dst.data_ptr(), dt, dh, positions.data_ptr(), inv_freq.data_ptr(), N, H,
+          width, dims, _code(src.dtype), _stream())
+    return dst
+
+
+def latent_kv_store(kv: torch.Tensor, norm_weight: torch.Tensor, eps: float, positions: torch.Tensor, inv_freq: torch.Tensor,
+                    slot_mapping: torch.Tensor, c_pages: torch.Tensor, r_pages: torch.Tensor) -> None:
+    """kv [N, C + R]: the RMS norm of its first C columns (times ``norm_weight``) goes to ``c_pages`` [P, 1, page, C], its
+    last R columns, turned pair by pair, to ``r_pages`` [P, 1, page, R], at ``slot_mapping`` (< 0: not stored)."""
+    N = kv.shape[0]
+    _check(c_pages, "c_pages", kv.dtype, (None, 1, None, None))
+    C = c_pages.shape[3]
+    _check(r_pages, "r_pages", kv.dtype, (c_pages.shape[0], 1, c_pages.shape[2], None))
+    R = r_pages.shape[3]
+    ks = _rows2d(kv, "kv", None, C + R)
+    _check(norm_weight, "norm_weight", torch.float32, (C,))
+    _check(positions, "positions", torch.int32, (N,))
+    _check(slot_mapping, "slot_mapping", torch.int32, (N,))
+    _check(inv_freq, "inv_freq", torch.float32)
+    _call("ms_latent_kv_store", kv.data_ptr(), ks, norm_weight.data_ptr(), float(eps), positions.data_ptr(),
+          inv_freq.data_ptr(), slot_mapping.data_ptr(), c_pages.data_ptr(), r_pages.data_ptr(), N, C, R,
+          2 * inv_freq.numel(), _code(kv.dtype), _stream())
+
+
+def latent_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, scale: float, window: Optional[int] = None,
+                     sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[n, h] = sum_j p_j c_j over the keys j visible to token n (the last ``window`` up to itself), with
+    p = exp(s_j) / (sum_i exp(s_i) + exp(sink[h])) and s_j = scale * q[n, h] . [c_j ; kr_j].  q [N, H, C + R] and out
+    [N, H, C] views; ``kv``: a KVView whose pages are "c" [P, 1, page, C] and "kr" [P, 1, page, R]."""
+    c_pages, r_pages = kv.pages["c"], kv.pages["kr"]
+    _check(c_pages, "c_pages", q.dtype, (None, 1, None, None))
+    P, _, page_size, C = c_pages.shape
+    _check(r_pages, "r_pages", q.dtype, (P, 1, page_size, None))
+    R = r_pages.shape[3]
+    N, H, width = q.shape
+    if width != C + R:
+        raise ValueError(f"queries of width {width} against keys of {C} + {R}")
+    qt, qh = _heads3d(q, "q")
+    ot, oh = _heads3d(out, "out", q.dtype)
+    if tuple(out.shape) != (N, H, C):
+        raise ValueError(f"out must be {[N, H, C]}, got {list(out.shape)}")
+    _check(kv.block_table, "block_table", torch.int32)
+    _check(ctx.token_req, "token_req", torch.int32, (N,))
+    _check(ctx.positions, "positions", torch.int32, (N,))
+    if kv.table_rows is not None:
+        _check(kv.table_rows, "table_rows", torch.int32)
+    if sink is not None:
+        _check(sink, "sink", torch.float32, (H,))
+    _call("ms_latent_attention", q.data_ptr(), qt, qh, c_pages.data_ptr(), r_pages.data_ptr(), kv.block_table.data_ptr(),
+          kv.block_table.shape[1], _ptr(kv.table_rows), _ptr(ctx.n_live_tokens), ctx.token_req.data_ptr(),
+          ctx.positions.data_ptr(), _ptr(sink), out.data_ptr(), ot, oh, N, H, C, R, page_size, P, float(scale),
+          int(window or 0), _code(q.dtype), _stream())
+    return out

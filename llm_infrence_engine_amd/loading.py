@@ -26,7 +26,11 @@ def load_model(model_dir, dtype: str = "bfloat16", device: str = "cuda:0") -> Mo
     if not torch.cuda.is_available():
         raise RuntimeError("no GPU is visible to this process; the engine has no CPU path")
     config = load_config(model_dir)
+    reader = CheckpointReader(model_dir)
+    if hasattr(config, "with_tensor_shapes"):     # sizes that config.json leaves to the tensors' shapes
+        names = set(reader.names())
+        config = config.with_tensor_shapes(lambda name: reader.shape(name) if name in names else None)
     model = Model(config.to_spec())
     model.config = config
-    model.load(CheckpointReader(model_dir), Runtime(dev, DTYPES[dtype]))
+    model.load(reader, Runtime(dev, DTYPES[dtype]))
     return model

@@ -7,6 +7,7 @@ it is in.  Five kinds are chosen layer by layer:
 ``PositionEncoding``  encode_and_store(qkv, nh, nkv, d, ctx, kv)                 (belongs to a mixer)
 ``Mixer``             forward(h, ctx, kv, state) -> [N, hidden]                  (attention here)
 ``FeedForward``       forward(h, ctx) -> [N, hidden]
+``SequenceFilter``    forward(h, ctx, state) -> [N, hidden]                      (a map over time before a part's input)
                       (both also forward_residual(..., x): add into the residual stream x and return None,
                       or return the addend; the default returns forward's result)
 ``Block``             forward(x, pending, ctx, kv, state) -> pending             (the arrangement; it names the parts it takes)
@@ -79,12 +80,12 @@ def KVNeed(num_kv_heads: int, head_dim: int, window: Optional[int] = None,
 
 @dataclass(frozen=True)
 class StateNeed:
-    """State of fixed size per request: one tensor of ``shape`` and ``dtype`` in a slot that the request holds
-    from admission to its end.  The slot is zero when the request's first portion runs.  A mixer that keeps
-    several such tensors returns a tuple of these."""
+    """State of fixed size per request: one tensor of ``shape`` and ``dtype`` (None: the type of the run's
+    activations) in a slot that the request holds from admission to its end.  The slot is zero when the request's
+    first portion runs.  A mixer that keeps several such tensors returns a tuple of these."""
 
     shape: Tuple[int, ...]
-    dtype: torch.dtype = torch.float32
+    dtype: Optional[torch.dtype] = torch.float32
 
 
 @dataclass
@@ -249,6 +250,18 @@ class Mixer(Part):
         return self.forward(h, ctx, kv, state)
 
 
+class SequenceFilter(Part):
+    """A small map over time that a block lays before a part's input (a short causal convolution, say): it sees
+    the step's tokens in order and keeps what it needs of a request's past in a state slot of its own."""
+
+    def state_need(self):
+        """None, or a ``StateNeed``."""
+        return None
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, state: Optional[StateView]) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class FeedForward(Part):
     accepts_lazy_norm = False
 
@@ -346,15 +359,37 @@ class Block(Part):
                       {k[len(prefix):]: v for k, v in kv.transposed.items() if k.startswith(prefix)},
                       kv.block_table, kv.slot_mapping, kv.store, kv.window, kv.table_rows)
 
+    def _state_needs(self):
+        """Per part that keeps state, in the order of ``takes``: (part name, its needs as a list)."""
+        out = []
+        for name, p in self.built.items():
+            if isinstance(p, (Mixer, SequenceFilter)):
+                n = p.state_need()
+                if n is not None:
+                    out.append((name, list(n) if isinstance(n, (tuple, list)) else [n]))
+        return out
+
     def state_need(self):
-        needs = []
-        for m in self.mixers():
-            n = m.state_need()
-            if n is not None:
-                needs.extend(n if isinstance(n, (tuple, list)) else [n])
+        needs = [n for _, ns in self._state_needs() for n in ns]
         if not needs:
             return None
         return needs[0] if len(needs) == 1 else tuple(needs)
+
+    def state_of(self, name: str, state: Optional[StateView]) -> Optional[StateView]:
+        """The part ``name``'s own share of the run's state tensors, shaped as the part declared it (one tensor,
+        or a tuple for several); the whole view when one part of the layer keeps state."""
+        per_part = self._state_needs()
+        if state is None or len(per_part) <= 1:
+            return state if any(n == name for n, _ in per_part) else None
+        slots = state.slots if isinstance(state.slots, (tuple, list)) else (state.slots,)
+        at = 0
+        for n, ns in per_part:
+            if n == name:
+                mine = tuple(slots[at:at + len(ns)])
+                declared = self.built[n].state_need()
+                return StateView(mine if isinstance(declared, (tuple, list)) else mine[0])
+            at += len(ns)
+        return None
 
     def graph_safe(self):
         return weakest(p.graph_safe for p in self.built.values() if p is not None)
@@ -388,7 +423,7 @@ class Head(Part):
 
 # ------------------------------------------------------------------------------------------------ registries
 _REGISTRIES: Dict[str, Dict[str, type]] = {
-    "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {}, "embedding": {}, "head": {},
+    "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "filter": {}, "block": {}, "embedding": {}, "head": {},
 }
 
 

@@ -6,6 +6,7 @@ it as an epilogue) or hands the addend on, and the sum is fused into the norm th
 own last addend on as ``pending``."""
 from __future__ import annotations
 
+from ..kernels import ops
 from .base import Block, register_part
 
 
@@ -21,4 +22,29 @@ class PreNormResidual(Block):
         return self.feed_forward.forward_residual(norm(x, delta=a), ctx, x)
 
 
+class ParallelResidual(Block):
+    """x <- x + mixer(f(norm1(x))) + feed_forward(norm2(x)): both branches read the same x.  ``input_filter``
+    (optional) is a map over time laid before the mixer's input, f; without a feed-forward the layer is
+    x <- x + mixer(f(norm1(x)))."""
+
+    takes = {"position": "position", "mixer_norm": "norm", "input_filter": "filter", "mixer": "mixer",
+             "feed_forward_norm": "norm", "feed_forward": "feed_forward"}
+    optional = ("position", "input_filter", "feed_forward_norm", "feed_forward")
+
+    def forward(self, x, pending, ctx, kv, state):
+        h = self.mixer_norm.forward(x, delta=pending)          # x now holds the sum both branches read
+        h2 = self.feed_forward_norm.forward(x) if self.feed_forward is not None else None
+        if self.input_filter is not None:
+            h = self.input_filter.forward(h, ctx, self.state_of("input_filter", state))
+        a = self.mixer.forward_residual(h, ctx, kv, self.state_of("mixer", state), x)
+        if self.feed_forward is None:
+            return a
+        b = self.feed_forward.forward_residual(h2, ctx, x)
+        if a is not None and b is not None:
+            ops.residual_add(x, a)
+            return b
+        return a if b is None else b
+
+
 register_part("block", "pre_norm_residual", PreNormResidual)
+register_part("block", "parallel_residual", ParallelResidual)

@@ -1,0 +1,96 @@
+"""The gated delta rule with one decay per head and key channel, as a mixer without a cache of keys.
+
+h -> q, k (kv_heads x dim), v (heads x vdim), each through a short causal convolution over time and SiLU; q and k
+made unit vectors per head (q also times dim^-1/2); beta = sigmoid(W_b h); the decay
+g = exp(-exp(A_log) * softplus(W_a2 W_a1 h + dt_bias)), one number per head and key channel.  Per head, with the
+state S [dim, vdim] carried from token to token in float:
+
+    S <- g * S (row i by g_i);  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+
+so the read-out sees the token's own write.  o is divided by its root mean square per head, scaled by a weight shared
+by the heads and gated by sigmoid(W_g2 W_g1 h); then the output projection.  Head i reads q/k head i // (heads //
+kv_heads).  State per request: the convolution's last taps - 1 inputs and S."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import linear, ops
+from ..weights.spec import TensorSpec
+from .base import Mixer, StateNeed, register_part
+
+
+def _rows(t: torch.Tensor, lo: int, hi: int) -> torch.Tensor:
+    """Columns lo..hi of ``t`` as the input of a product: the slice itself where a kernel takes it as it lies."""
+    s = t[:, lo:hi]
+    if t.dtype == torch.float32 or (t.shape[0] <= ops.SKINNY_MAX_ROWS and ops.skinny_ok(s, s)):
+        return s
+    return s.contiguous()
+
+
+class GatedDelta(Mixer):
+    graph_safe = True      # its kernels walk the requests from the step's device tensors
+
+    def __init__(self, prefix: str, position, hidden_size: int, heads: int, kv_heads: int, dim: int, vdim: int, taps: int,
+                 decay_rank: int, gate_rank: int, eps: float):
+        if heads % kv_heads:
+            raise ValueError(f"{heads} heads cannot share {kv_heads} query/key heads")
+        if not 1 <= taps <= ops.MAX_CONV_TAPS:
+            raise ValueError(f"a short convolution has 1 to {ops.MAX_CONV_TAPS} taps, got {taps}")
+        if dim > 512:
+            raise ValueError(f"key size {dim} is not supported: the kernel holds a column of the state in registers, up to 512 rows")
+        self.prefix, self.hidden_size = prefix, hidden_size
+        self.heads, self.kv_heads, self.dim, self.vdim, self.taps = heads, kv_heads, dim, vdim, taps
+        self.decay_rank, self.gate_rank, self.eps = decay_rank, gate_rank, float(eps)
+        self.qk, self.vw = kv_heads * dim, heads * vdim
+
+    # ---- weights
+    def tensor_specs(self):
+        p, W = self.prefix, self.hidden_size
+        H, D = self.heads, self.dim
+        specs = []
+        for name, rows in (("q", self.qk), ("k", self.qk), ("v", self.vw)):
+            specs += [TensorSpec(p + name, (rows, W)), TensorSpec(p + name + ".conv", (rows, self.taps), "bias")]
+        specs += [TensorSpec(p + "b", (H, W)), TensorSpec(p + "A_log", (H,), "bias"),
+                  TensorSpec(p + "norm", (self.vdim,), "norm"),
+                  TensorSpec(p + "a1", (self.decay_rank, W)), TensorSpec(p + "a2", (H * D, self.decay_rank)),
+                  TensorSpec(p + "dt_bias", (H * D,), "bias"),
+                  TensorSpec(p + "g1", (self.gate_rank, W)), TensorSpec(p + "g2", (self.vw, self.gate_rank)),
+                  TensorSpec(p + "o", (W, self.vw))]
+        return specs
+
+    def load(self, get, rt):
+        self.rt = rt
+        t = {s.name[len(self.prefix):]: get(s) for s in self.tensor_specs()}
+        # one product for everything that reads h: q | k | v | a1 | g1 | b
+        self.w_in = linear.prepare_weight(torch.cat([t["q"], t["k"], t["v"], t["a1"], t["g1"], t["b"]], dim=0))
+        self.conv_w = torch.cat([t["q.conv"], t["k.conv"], t["v.conv"]], dim=0).contiguous()
+        self.w_a2, self.w_g2, self.w_o = (linear.prepare_weight(t[n]) for n in ("a2", "g2", "o"))
+        self.A_log, self.dt_bias, self.norm_w = t["A_log"], t["dt_bias"], t["norm"]
+
+    # ---- state
+    def state_need(self):
+        return (StateNeed((max(1, self.taps - 1), 2 * self.qk + self.vw), None),
+                StateNeed((self.heads, self.dim, self.vdim), torch.float32))
+
+    # ---- step
+    def forward(self, h, ctx, kv, state):
+        return self.forward_residual(h, ctx, kv, state, None)
+
+    def forward_residual(self, h, ctx, kv, state, x):
+        conv_state, S = state.slots
+        N = ctx.num_tokens
+        cw = 2 * self.qk + self.vw
+        a_at, g_at = cw, cw + self.decay_rank
+        b_at = g_at + self.gate_rank
+        proj = linear.linear(h, self.w_in)
+        qkv = ops.short_conv(proj[:, :cw], self.conv_w, conv_state, ctx, self.rt.empty(N, cw), ops.CONV_SILU)
+        a = linear.linear(_rows(proj, a_at, g_at), self.w_a2, out_dtype=torch.float32)
+        gate = linear.linear(_rows(proj, g_at, b_at), self.w_g2)
+        o = self.rt.empty(N, self.vw, dtype=torch.float32)
+        ops.gated_delta(qkv[:, :self.qk], qkv[:, self.qk:2 * self.qk], qkv[:, 2 * self.qk:], a, proj[:, b_at:],
+                        self.A_log, self.dt_bias, S, ctx, o, self.heads, self.kv_heads, self.dim, self.vdim)
+        y = ops.gated_head_norm(o, self.norm_w, gate, self.rt.empty(N, self.vw), self.heads, self.vdim, self.eps)
+        return linear.linear_residual(y, self.w_o, None, x)
+
+
+register_part("mixer", "gated_delta", GatedDelta)

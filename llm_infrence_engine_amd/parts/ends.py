@@ -11,11 +11,11 @@ from .base import Embedding, Head, register_part
 
 
 class TokenEmbedding(Embedding):
-    def __init__(self, prefix: str, vocab_size: int, hidden_size: int):
-        self.prefix, self.vocab_size, self.hidden_size = prefix, vocab_size, hidden_size
+    def __init__(self, prefix: str, vocab_size: int, hidden_size: int, name: str = "weight"):
+        self.prefix, self.vocab_size, self.hidden_size, self.name = prefix, vocab_size, hidden_size, name
 
     def tensor_specs(self):
-        return [TensorSpec(self.prefix + "weight", (self.vocab_size, self.hidden_size))]
+        return [TensorSpec(self.prefix + self.name, (self.vocab_size, self.hidden_size))]
 
     def load(self, get, rt):
         self.rt = rt
@@ -29,16 +29,16 @@ class TokenEmbedding(Embedding):
 class LMHead(Head):
     accepts_lazy_norm = True
 
-    def __init__(self, prefix: str, hidden_size: int, vocab_size: int, tied_to=None):
-        self.prefix, self.hidden_size, self.vocab_size, self.tied_to = prefix, hidden_size, vocab_size, tied_to
+    def __init__(self, prefix: str, hidden_size: int, vocab_size: int, tied_to=None, name: str = "weight"):
+        self.prefix, self.hidden_size, self.vocab_size, self.tied_to, self.name = prefix, hidden_size, vocab_size, tied_to, name
 
     def tensor_specs(self):
-        name = self.tied_to or self.prefix + "weight"
+        name = self.tied_to or self.prefix + self.name
         return [TensorSpec(name, (self.vocab_size, self.hidden_size))]
 
     def ignorable(self):
         """A tied head ignores a copy of its own that the checkpoint may still carry."""
-        return [self.prefix + "weight"] if self.tied_to else []
+        return [self.prefix + self.name] if self.tied_to else []
 
     def load(self, get, rt):
         self.rt = rt

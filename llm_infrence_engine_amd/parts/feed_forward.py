@@ -3,7 +3,9 @@ Gate and up are one packed matrix product (rows interleaved so that the activati
 epilogue); the activation is float."""
 from __future__ import annotations
 
-from ..kernels import linear
+import torch
+
+from ..kernels import linear, ops
 from ..weights.spec import TensorSpec
 from .base import FeedForward, register_part
 
@@ -32,4 +34,33 @@ class SwiGLU(FeedForward):
         return linear.linear_residual(linear.linear_swiglu(h, self.w_gate_up), self.w_down, None, x)
 
 
+class DenseAct(FeedForward):
+    """down(act(up(x))), no biases.  ``activation``: "xielu", with two learned numbers (p, q) in the tensor ``act``:
+    z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2."""
+
+    ACTIVATIONS = ("xielu",)
+
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "xielu"):
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"no activation {activation!r}; there are {', '.join(self.ACTIVATIONS)}")
+        self.prefix, self.hidden_size, self.intermediate_size, self.activation = prefix, hidden_size, intermediate_size, activation
+
+    def tensor_specs(self):
+        p, H, I = self.prefix, self.hidden_size, self.intermediate_size
+        return [TensorSpec(p + "up", (I, H)), TensorSpec(p + "down", (H, I)), TensorSpec(p + "act", (2,), "bias")]
+
+    def load(self, get, rt):
+        self.rt = rt
+        up, down, act = (get(s) for s in self.tensor_specs())
+        self.w_up, self.w_down, self.act = linear.prepare_weight(up), linear.prepare_weight(down), act
+
+    def forward(self, h, ctx):
+        return self.forward_residual(h, ctx, None)
+
+    def forward_residual(self, h, ctx, x):
+        u = linear.linear(h, self.w_up)
+        return linear.linear_residual(ops.xielu(u, self.act, torch.empty_like(u)), self.w_down, None, x)
+
+
 register_part("feed_forward", "swiglu", SwiGLU)
+register_part("feed_forward", "dense_act", DenseAct)

@@ -13,7 +13,7 @@ import torch
 from ..config.spec import ModelSpec
 from ..weights.reader import CheckpointReader, place
 from ..weights.spec import TensorSpec
-from . import attention, blocks, ends, feed_forward, norms, positions  # noqa: F401  (register the built-in parts)
+from . import attention, blocks, delta, ends, feed_forward, filters, latent, norms, positions  # noqa: F401  (register the built-in parts)
 from .base import KVView, Runtime, StateView, StepContext, build_part, part_class, weakest
 
 
@@ -51,7 +51,7 @@ class Model:
         return out
 
     def ignorable_tensors(self) -> List[str]:
-        return list(getattr(self.head, "ignorable", lambda: [])())
+        return list(getattr(self.head, "ignorable", lambda: [])()) + list(self.spec.ignorable)
 
     def load(self, reader: CheckpointReader, rt: Runtime) -> "Model":
         reader.check(self.tensor_specs(), self.ignorable_tensors())

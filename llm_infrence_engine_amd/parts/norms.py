@@ -1,4 +1,6 @@
-"""RMS norm: y = weight * x * rsqrt(mean(x^2) + eps), computed in float on the float residual stream.
+"""RMS norm: y = (offset + weight) * x * rsqrt(mean(x^2) + eps), computed in float on the float residual stream.
+``offset`` is 0 for a scale stored as it is and 1 for one stored around zero; the sum is formed once, in float,
+when the weights are loaded.
 
 The reference computes the reduction in float, casts back and multiplies by the weight in the model's
 type (src/miniserve/model.py:69-73); here the weight is applied in float too and the result is rounded once.
@@ -13,15 +15,18 @@ from .base import Norm, register_part
 
 
 class RMSNorm(Norm):
-    def __init__(self, prefix: str, size: int, eps: float):
-        self.prefix, self.size, self.eps = prefix, size, eps
+    def __init__(self, prefix: str, size: int, eps: float, offset: float = 0.0, name: str = "weight"):
+        self.prefix, self.size, self.eps, self.offset, self.name = prefix, size, eps, float(offset), name
 
     def tensor_specs(self):
-        return [TensorSpec(self.prefix + "weight", (self.size,), "norm")]
+        # a scale stored around zero is drawn around zero by the random-weights mode too
+        return [TensorSpec(self.prefix + self.name, (self.size,), "bias" if self.offset else "norm")]
 
     def load(self, get, rt):
         self.rt = rt
         self.weight = get(self.tensor_specs()[0])
+        if self.offset:
+            self.weight = (self.weight + self.offset).contiguous()
 
     def forward(self, x, delta=None, rows=None, write_back=True):
         n = x.shape[0] if rows is None else rows.numel()

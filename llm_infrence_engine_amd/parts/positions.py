@@ -62,5 +62,26 @@ class NoPosition(PositionEncoding):
                            kv.v_pages, kv.v_transposed)
 
 
+class RotaryPairs(PositionEncoding):
+    """Rotary encoding with neighbouring entries paired: of a vector's first ``dims`` entries, entry 2i and entry
+    2i + 1 turn by position * theta^(-2i/dims); the rest pass unchanged.  It turns whatever slice of a vector its
+    mixer hands it (``rotate``); angles, sines and cosines are float."""
+
+    def __init__(self, prefix: str, width: int, dims: int, theta: float):
+        if dims % 2 or not 0 <= dims <= width:
+            raise ValueError(f"{dims} rotated entries must be even and within the vector's width {width}")
+        self.width, self.dims, self.theta = width, dims, float(theta)
+
+    def load(self, get, rt):
+        self.rt = rt
+        i = torch.arange(0, self.dims, 2, dtype=torch.float64)
+        self.inv_freq = (self.theta ** (-i / max(1, self.dims))).to(torch.float32).to(rt.device)
+
+    def rotate(self, src, dst, ctx):
+        """dst[n, h] = src[n, h] turned by the position of token n; [N, heads, width] views, dst may be src."""
+        return ops.rotary_pairs(src, dst, ctx.positions, self.inv_freq)
+
+
 register_part("position", "rotary_half", RotaryHalf)
+register_part("position", "rotary_pairs", RotaryPairs)
 register_part("position", "none", NoPosition)
