@@ -74,7 +74,7 @@ __global__ void short_conv_update_kernel(const T* __restrict__ x, size_t x_strid
 // g = exp(-exp(A_log_h) * softplus(a + dt_bias)).  Column j of S depends on no other column, so a column is
 // held in the registers of LPC neighbouring lanes (DPT rows each) for the whole portion.  Tokens are staged a
 // chunk at a time: the chunk's q, k (normalised), g, beta and v are worked out by all threads in parallel into
-// LDS, then the chunk's tokens are walked in order.
+// LDS, then the chunk's tokens are walked in order.  The chunk is as long as LDS allows, up to 16 tokens.
 constexpr int DELTA_CHUNK = 16;
 
 template <typename T, int DPT>
@@ -83,14 +83,14 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
                    const float* __restrict__ a, const T* __restrict__ b, size_t b_stride,
                    const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ state,
                    const int* __restrict__ q_start, const int* __restrict__ state_slots, float* __restrict__ out,
-                   int H, int G, int D, int E, int lpc, int cols_per_block) {
+                   int H, int G, int D, int E, int lpc, int cols_per_block, int chunk) {
   extern __shared__ __align__(16) float lds[];
-  const int Dp = DPT * lpc;                       // padded key size
-  float* qs = lds;                                // [CHUNK][Dp]
-  float* ks = qs + DELTA_CHUNK * Dp;
-  float* gs = ks + DELTA_CHUNK * Dp;
-  float* vs = gs + DELTA_CHUNK * Dp;              // [CHUNK][cols_per_block]
-  float* bs = vs + DELTA_CHUNK * cols_per_block;  // [CHUNK]
+  const int Dp = DPT * lpc;                 // padded key size
+  float* qs = lds;                          // [chunk][Dp]
+  float* ks = qs + chunk * Dp;
+  float* gs = ks + chunk * Dp;
+  float* vs = gs + chunk * Dp;              // [chunk][cols_per_block]
+  float* bs = vs + chunk * cols_per_block;  // [chunk]
   const int r = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * cols_per_block;
   const int kvh = h / (H / G);
   const int s0 = q_start[r], L = q_start[r + 1] - s0;
@@ -108,8 +108,8 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
   const float rate = expf(A_log[h]);
   const float q_scale = 1.0f / sqrtf((float)D);
 
-  for (int c0 = 0; c0 < L; c0 += DELTA_CHUNK) {
-    const int cn = min(DELTA_CHUNK, L - c0);
+  for (int c0 = 0; c0 < L; c0 += chunk) {
+    const int cn = min(chunk, L - c0);
     __syncthreads();   // the chunk before is done with the staging area
     for (int t = wave; t < cn; t += nwaves) {        // a wave normalises a token's q and k
       const size_t n = (size_t)(s0 + c0 + t);
@@ -258,13 +258,16 @@ extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long 
   threads = threads >= 256 ? 256 : ((threads + MS_WAVE - 1) / MS_WAVE) * MS_WAVE;
   const int cols = threads / lpc;
   dim3 grid((vdim + cols - 1) / cols, heads, n_requests), block(threads);
-  const size_t lds = (size_t)DELTA_CHUNK * (3 * (size_t)dpt * lpc + cols + 1) * sizeof(float);
+  int chunk = DELTA_CHUNK;
+  const size_t per_token = (3 * (size_t)dpt * lpc + cols + 1) * sizeof(float);
+  while (chunk > 1 && chunk * per_token > 65536) chunk /= 2;
+  const size_t lds = chunk * per_token;
   if (lds > 65536) return MS_UNSUPPORTED;
 #define LAUNCH(T, DPT)                                                                                                  \
   gated_delta_kernel<T, DPT><<<grid, block, lds, stream>>>((const T*)q, (const T*)k, (const T*)v, (size_t)qkv_stride, \
                                                            a, (const T*)b, (size_t)b_stride, A_log, dt_bias, state,   \
                                                            q_start, state_slots, out, heads, kv_heads, dim, vdim,     \
-                                                           lpc, cols)
+                                                           lpc, cols, chunk)
 #define BY_DPT(T)                                                                                                       \
   do {                                                                                                                  \
     if (dpt == 8) LAUNCH(T, 8);                                                                                         \

@@ -99,9 +99,19 @@ def rotate_interleaved(x: torch.Tensor, positions: torch.Tensor, dims: int, base
 
 
 # --------------------------------------------------------------------------- feed-forward
-def dense_ff(h, w, prefix):
+def same(x):
+    return x
+
+
+def rounder(act_dtype):
+    """x as an engine that stores activations in ``act_dtype`` would hold it (None: exact).  Used only to measure
+    how far a faithful reduced-precision computation strays from the exact one."""
+    return same if act_dtype is None else (lambda x: x.to(act_dtype).to(x.dtype))
+
+
+def dense_ff(h, w, prefix, rd=same):
     act = w[prefix + "act"]
-    return xielu(h @ w[prefix + "up"].T, act[0], act[1]) @ w[prefix + "down"].T
+    return rd(rd(xielu(rd(h @ w[prefix + "up"].T), act[0], act[1])) @ w[prefix + "down"].T)
 
 
 # --------------------------------------------------------------------------- the delta-rule mixer
@@ -120,44 +130,45 @@ def delta_rule(q, k, v, g, beta):
     return out
 
 
-def channel_delta(h, w, prefix, m, eps):
-    """h [T, W]; ``m`` the mixer's sizes (heads, kv_heads, dim, vdim)."""
+def channel_delta(h, w, prefix, m, eps, rd=same):
+    """h [T, W]; ``m`` the mixer's sizes (heads, kv_heads, dim, vdim).  ``rd`` rounds what an engine would store in
+    its activations' type (the recurrence itself and what enters it beside q, k, v stay exact)."""
     T = h.shape[0]
     H, G, D, E = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
 
     def branch(name):
-        return F.silu(causal_conv(h @ w[prefix + name].T, w[prefix + name + ".conv"]))
+        return rd(F.silu(causal_conv(rd(h @ w[prefix + name].T), w[prefix + name + ".conv"])))
 
     q = branch("q").reshape(T, G, D)
     k = branch("k").reshape(T, G, D)
     v = branch("v").reshape(T, H, E)
     q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
     k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
-    beta = torch.sigmoid(h @ w[prefix + "b"].T)                                   # [T, H]
-    a = (h @ w[prefix + "a1"].T) @ w[prefix + "a2"].T + w[prefix + "dt_bias"]       # [T, H*D]
+    beta = torch.sigmoid(rd(h @ w[prefix + "b"].T))                               # [T, H]
+    a = rd(h @ w[prefix + "a1"].T) @ w[prefix + "a2"].T + w[prefix + "dt_bias"]     # [T, H*D]
     rate = torch.exp(w[prefix + "A_log"])                                          # [H]
     g = torch.exp(-rate[None, :, None] * F.softplus(a.reshape(T, H, D)))
-    gate = torch.sigmoid((h @ w[prefix + "g1"].T) @ w[prefix + "g2"].T).reshape(T, H, E)
+    gate = torch.sigmoid(rd(rd(h @ w[prefix + "g1"].T) @ w[prefix + "g2"].T)).reshape(T, H, E)
     heads = []
     for i in range(H):
         j = i // (H // G)
         o = delta_rule(q[:, j], k[:, j], v[:, i], g[:, i], beta[:, i])
         heads.append(plain_norm(o, w[prefix + "norm"], eps) * gate[:, i])
-    return torch.cat(heads, dim=-1) @ w[prefix + "o"].T
+    return rd(rd(torch.cat(heads, dim=-1)) @ w[prefix + "o"].T)
 
 
 # --------------------------------------------------------------------------- latent attention
-def latent_attention(h, w, prefix, m, eps):
+def latent_attention(h, w, prefix, m, eps, rd=same):
     """h [T, W]; ``m``: heads, dim (unrotated), rot_dim, vdim, kv_rank, rot {base, dims}, mask {size}, scale."""
     T = h.shape[0]
     H, D, R, E, C = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
     pos = torch.arange(T)
-    cq = plain_norm(h @ w[prefix + "dq"].T, w[prefix + "dq.norm"], eps)
-    q = (cq @ w[prefix + "uq"].T).reshape(T, H, D + R)
+    cq = rd(plain_norm(rd(h @ w[prefix + "dq"].T), w[prefix + "dq.norm"], eps))
+    q = rd(cq @ w[prefix + "uq"].T).reshape(T, H, D + R)
     q_flat, q_rot = q[..., :D], rotate_interleaved(q[..., D:], pos, m["rot"]["dims"], m["rot"]["base"])
-    kv = h @ w[prefix + "dkv"].T
-    c = plain_norm(kv[:, :C], w[prefix + "dkv.norm"], eps)
-    k_rot = rotate_interleaved(kv[:, C:], pos, m["rot"]["dims"], m["rot"]["base"])        # [T, R], shared by heads
+    kv = rd(h @ w[prefix + "dkv"].T)
+    c = rd(plain_norm(kv[:, :C], w[prefix + "dkv.norm"], eps))
+    k_rot = rd(rotate_interleaved(kv[:, C:], pos, m["rot"]["dims"], m["rot"]["base"]))    # [T, R], shared by heads
     k_flat = (c @ w[prefix + "uk"].T).reshape(T, H, D)
     v = (c @ w[prefix + "uv"].T).reshape(T, H, E)
     window = (m.get("mask") or {}).get("size")
@@ -170,27 +181,30 @@ def latent_attention(h, w, prefix, m, eps):
             top = torch.maximum(s.max(), sink)
             e = torch.exp(s - top)
             out[t, i] = (e[:, None] * v[lo:t + 1, i]).sum(0) / (e.sum() + torch.exp(sink - top))
-    gate = torch.sigmoid(h @ w[prefix + "g"].T)
-    return (out.reshape(T, H * E) * gate) @ w[prefix + "o"].T
+    gate = torch.sigmoid(rd(h @ w[prefix + "g"].T))
+    return rd(rd(out.reshape(T, H * E) * gate) @ w[prefix + "o"].T)
 
 
 MIXERS = {"channel_delta": channel_delta, "latent_attention": latent_attention}
 
 
 # --------------------------------------------------------------------------- the model
-def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out=None) -> torch.Tensor:
-    """Logits [T, vocab] of one sequence.  ``layers_out``: a list that receives the residual stream after every layer."""
+def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out=None, act_dtype=None) -> torch.Tensor:
+    """Logits [T, vocab] of one sequence.  ``layers_out``: a list that receives the residual stream after every layer.
+    ``act_dtype``: round the activations between the products as an engine of that type would (the residual stream,
+    the norms' and recurrences' own arithmetic stay exact)."""
+    rd = rounder(act_dtype)
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in w.items()}
     eps = cfg["norm"]["eps"]
     x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)]
     for i, layer in enumerate(cfg["layers"]):
         p = f"l{i}."
-        n = offset_norm(x, w[p + "norm1"], eps)
-        h = n + causal_conv(n, w[p + "canon1"])
-        y = MIXERS[layer["type"]](h, w, p + "mix.", layer["mixer"], eps)
+        n = rd(offset_norm(x, w[p + "norm1"], eps))
+        h = rd(n + causal_conv(n, w[p + "canon1"]))
+        y = MIXERS[layer["type"]](h, w, p + "mix.", layer["mixer"], eps, rd)
         if layer.get("mlp") is not None:
-            y = y + dense_ff(offset_norm(x, w[p + "norm2"], eps), w, p + "mlp.")
+            y = y + dense_ff(rd(offset_norm(x, w[p + "norm2"], eps)), w, p + "mlp.", rd)
         x = x + y
         if layers_out is not None:
             layers_out.append(x.clone())
-    return offset_norm(x, w["final.norm"], eps) @ w["head"].T
+    return rd(offset_norm(x, w["final.norm"], eps)) @ w["head"].T
