@@ -18,6 +18,11 @@ the same way, all their layers with weights drawn on the GPU: ``shapes["7b"]`` (
 2,048-token prompt, a queue of 64 requests with prompts of 128 to 4,096 tokens and 256 decoded each) and
 ``shapes["32b"]`` (the prompt, decode at batch 1, 8 and 64 after 1,024-token prompts); ``--no-shapes`` leaves
 them out.  ``--only sample`` times the sampler alone at the real vocabulary.
+
+``--design gemadra`` measures another design instead: the Gemadra decoder (delta-rule and latent-attention layers in
+turn) beside the Qwen2 decoder at the same width, depth and feed-forward weights, a 2,048-token prompt in one step
+and decode steps at batch 8 and 64, at the widths of the 0.5B and the 7B shape (``--design-layers`` layers each,
+random weights, bfloat16); one JSON line, ``sizes[width][design]``.
 """
 from __future__ import annotations
 
@@ -240,8 +245,69 @@ def run_serving(eng_mod, model, vocab, seed, n_requests=64, new_tokens=256, lo=1
             "wasted_row_fraction": round(s["wasted_row_fraction"], 4)}
 
 
+def generic_costs(model, cfg_dict=None):
+    """(bytes of the matrices a decode step reads, matrix multiply-adds a token) from the model's own tensor list:
+    every matrix but the embedding table, whose rows are gathered."""
+    embed = {s.name for s in model.embedding.tensor_specs()} - {s.name for s in model.head.tensor_specs()}
+    macs = sum(s.shape[0] * s.shape[1] for s in model.tensor_specs()
+               if s.role == "matrix" and len(s.shape) == 2 and s.name not in embed)
+    return 2 * macs, macs
+
+
+def run_design(eng, a):
+    """Gemadra beside Qwen2 at equal width, depth and feed-forward weights."""
+    import gc
+
+    import torch
+
+    from llm_infrence_engine_amd.config import config_from_dict, preset
+
+    out = {"design": "gemadra", "beside": "qwen2", "layers": a.design_layers, "dtype": "bf16", "data": "synthetic",
+           "prefill_tokens": PREFILL_TOKENS, "prompt_len": a.prompt_len, "sizes": {}}
+    for size in a.design_sizes.split(","):
+        row = {}
+        for design, name in (("gemadra", "gemadra-" + size), ("qwen2", size)):
+            if a.design_only not in (None, design):
+                continue
+            d = preset(name)
+            if design == "gemadra":
+                d["layers"] = d["layers"][:a.design_layers]
+            else:
+                d["num_hidden_layers"] = a.design_layers
+            cfg = config_from_dict(d)
+            model = eng.load_random_model(cfg, seed=0, dtype="bfloat16", device="cuda:0")
+            vocab = model.spec.vocab_size
+            wbytes, macs = generic_costs(model)
+            r = {"matrix_weights_M": round(macs / 1e6, 1)}
+            if a.design_part in ("all", "prefill"):
+                pt = run_prefill(eng, model, vocab, seed=2, repeats=3)
+                r.update({"prefill_ms": round(pt * 1e3, 3), "prefill_tokens_per_s": round(PREFILL_TOKENS / pt, 1),
+                          "prefill_matrix_frac": round(2.0 * macs * PREFILL_TOKENS / pt / 1e12 / PEAK_TFLOPS["bf16"], 4)})
+            if a.design_part in ("all", "decode"):
+                for b in (8, 64):
+                    dt, _, _ = run_decode(eng, model, b, min(a.steps, 64), min(a.warmup, 8), vocab, seed=3 + b,
+                                          prompt_len=a.prompt_len)
+                    r.update({f"decode_b{b}_ms_per_step": round(dt * 1e3, 4), f"decode_b{b}_tokens_per_s": round(b / dt, 1),
+                              f"decode_b{b}_weights_frac": round(wbytes / dt / 1e9 / HBM_GBS, 4)})
+            row[design] = r
+            del model
+            gc.collect()
+            torch.cuda.empty_cache()
+        out["sizes"][size] = row
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--design", choices=["gemadra"], default=None,
+                    help="measure this design beside the Qwen2 decoder at equal sizes instead of the default workload")
+    ap.add_argument("--design-layers", type=int, default=4, help="layers of each model in a --design run")
+    ap.add_argument("--design-sizes", default="0.5b,7b", help="widths of a --design run (0.5b, 7b)")
+    ap.add_argument("--design-part", choices=["all", "prefill", "decode"], default="all",
+                    help="a --design run's prompt step or its decode steps alone (for profiles)")
+    ap.add_argument("--design-only", choices=["gemadra", "qwen2"], default=None,
+                    help="one of the two models of a --design run alone (for profiles)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
@@ -267,6 +333,8 @@ def main() -> int:
     import llm_infrence_engine_amd as eng
     from llm_infrence_engine_amd.config import config_from_dict, preset
 
+    if a.design:
+        return run_design(eng, a)
     shape = preset(a.shape)
     if a.layers is None:
         a.layers = shape["num_hidden_layers"]

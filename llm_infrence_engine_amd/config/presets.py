@@ -1,5 +1,6 @@
 """Named config.json contents for the random-weights mode: the shapes the published Qwen2.5 checkpoints
-have and the two tiny ones the tests use, so that ``--random-config 0.5b`` needs no file.  These are data
+have, the two tiny ones the tests use and two Gemadra shapes of the same widths, so that ``--random-config 0.5b``
+needs no file.  These are data
 of the kind a config.json holds; no part or kernel reads them.
 """
 from __future__ import annotations
@@ -20,7 +21,33 @@ PRESETS = {
 }
 
 
+
+
+def _gemadra(width, ff, layers, delta, latent, vocab=151936):
+    """``layers`` layers, the two mixers in turn (the delta rule first); ranks of the delta mixer's low-rank maps stated."""
+    d = {"type": "channel_delta", "mixer": dict(delta), "mlp": {"kind": "dense", "ff": ff}}
+    a = {"type": "latent_attention", "mixer": dict(latent), "mlp": {"kind": "dense", "ff": ff}}
+    return {"architecture": "Gemadra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "canon": {"taps": 4},
+            "layers": [dict(d) if i % 2 == 0 else dict(a) for i in range(layers)]}
+
+
+# Gemadra at the widths of the two smaller Qwen2.5 shapes, with a feed-forward of as many weights (two matrices of
+# 1.5 x the gated one's inner size) and mixers of a comparable number: for measurements beside those shapes
+PRESETS["gemadra-0.5b"] = _gemadra(
+    896, 7296, 24,
+    {"heads": 14, "kv_heads": 7, "dim": 64, "vdim": 64, "conv": 4, "decay_rank": 64, "gate_rank": 64},
+    {"heads": 14, "dim": 64, "rot_dim": 32, "vdim": 64, "kv_rank": 256, "q_rank": 384, "mask": {"size": 1024},
+     "rot": {"base": 10000.0, "dims": 32}, "scale": 96 ** -0.5})
+PRESETS["gemadra-7b"] = _gemadra(
+    3584, 28416, 28,
+    {"heads": 28, "kv_heads": 14, "dim": 128, "vdim": 128, "conv": 4, "decay_rank": 128, "gate_rank": 128},
+    {"heads": 28, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": 1536, "mask": {"size": 1024},
+     "rot": {"base": 10000.0, "dims": 64}, "scale": 192 ** -0.5}, vocab=152064)
+
+
 def preset(name: str) -> dict:
     if name not in PRESETS:
         raise KeyError(f"no preset {name!r}; there are {', '.join(sorted(PRESETS))}")
-    return dict(PRESETS[name])
+    import copy
+
+    return copy.deepcopy(PRESETS[name])
