@@ -41,6 +41,9 @@ class CachePools:
             for t in key.tensors:
                 flipped[t.name] = (t.transpose_at is not None and page_size % t.transpose_at == 0
                                    and t.transpose_in in (None, rt.dtype))
+                if t.only_transposed and not flipped[t.name]:
+                    del flipped[t.name]        # a copy that only the transposed layout is good for
+                    continue
                 inner = (t.width, page_size) if flipped[t.name] else (page_size, t.width)
                 tensors[t.name] = torch.zeros((len(runs), num_pages + 1, t.heads, *inner), dtype=rt.dtype, device=rt.device)
             self.pages.append(tensors)

@@ -180,12 +180,20 @@ int ms_rotary_pairs(const void* src, long long src_tok, long long src_head, void
                     long long dst_head, const int* positions, const float* inv_freq, int n_tokens, int heads, int width,
                     int dims, int dtype, hipStream_t stream);
 int ms_latent_kv_store(const void* kv, long long kv_stride, const float* norm_w, float eps, const int* positions,
-                       const float* inv_freq, const int* slots, void* c_pages, void* r_pages, int n_tokens, int C, int R,
-                       int dims, int dtype, hipStream_t stream);
+                       const float* inv_freq, const int* slots, void* c_pages, void* r_pages, void* ct_pages, int page_size,
+                       int n_tokens, int C, int R, int dims, int dtype, hipStream_t stream);
 int ms_latent_attention(const void* q, long long q_tok, long long q_head, const void* c_pages, const void* r_pages,
                         const int* block_table, int table_stride, const int* table_rows, const int* n_live_tokens,
                         const int* token_req, const int* positions, const float* sink, void* out, long long out_tok,
                         long long out_head, int n_tokens, int heads, int C, int R, int page_size, long long num_pages,
                         float scale, int window, int dtype, hipStream_t stream);
+
+// the same on the matrix cores (csrc/latent_attention_mfma.hip): bfloat16, sizes ms_latent_attention_mfma_supported says
+int ms_latent_attention_mfma_supported(int C, int R, int page_size);
+int ms_latent_attention_mfma(const void* q, long long q_tok, long long q_head, const void* c_pages, const void* r_pages,
+                             const void* ct_pages, const int* block_table, int table_stride, const int* table_rows,
+                             const int* q_start, const int* context_lens, const float* sink, void* out, long long out_tok,
+                             long long out_head, int n_requests, int max_q_len, int heads, int C, int R, int page_size,
+                             long long num_pages, float scale, int window, hipStream_t stream);
 
 }  // extern "C"

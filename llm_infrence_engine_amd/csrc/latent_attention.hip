@@ -98,11 +98,12 @@ __global__ void rms_norm_rows_kernel(const T* __restrict__ in, size_t in_stride,
 
 // ------------------------------------------------------------------------------------------------
 // kv [N, C + R]: c = rms_norm(kv[:, :C]) * w -> latent pages at the token's slot; kv[:, C:] rotated -> key-part pages.
+// Pages are [page][slot][entry] with one head.
 template <typename T>
 __global__ void latent_kv_store_kernel(const T* __restrict__ kv, size_t kv_stride, const float* __restrict__ w, float eps,
                                        const int* __restrict__ positions, const float* __restrict__ inv_freq,
                                        const int* __restrict__ slots, T* __restrict__ c_pages, T* __restrict__ r_pages,
-                                       int C, int R, int dims) {
+                                       T* __restrict__ ct_pages, int page_size, int C, int R, int dims) {
   __shared__ float red[16];
   const int n = blockIdx.x;
   const int slot = slots[n];
@@ -113,7 +114,14 @@ __global__ void latent_kv_store_kernel(const T* __restrict__ kv, size_t kv_strid
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)C + eps);
   T* cp = c_pages + (size_t)slot * C;
-  for (int i = threadIdx.x; i < C; i += blockDim.x) cp[i] = from_float<T>(to_float(x[i]) * inv * w[i]);
+  // ct_pages (may be null): the same latents once more as [page][entry][slot], for kernels that read them as a
+  // matrix operand with the keys along a row
+  T* tp = ct_pages ? ct_pages + (size_t)(slot / page_size) * page_size * C + slot % page_size : nullptr;
+  for (int i = threadIdx.x; i < C; i += blockDim.x) {
+    const T v = from_float<T>(to_float(x[i]) * inv * w[i]);
+    cp[i] = v;
+    if (tp) tp[(size_t)i * page_size] = v;
+  }
   const float pos = (float)positions[n];
   T* rp = r_pages + (size_t)slot * R;
   const T* xr = x + C;
@@ -262,17 +270,17 @@ extern "C" int ms_rotary_pairs(const void* src, long long src_tok, long long src
 }
 
 extern "C" int ms_latent_kv_store(const void* kv, long long kv_stride, const float* norm_w, float eps, const int* positions,
-                                  const float* inv_freq, const int* slots, void* c_pages, void* r_pages, int n_tokens,
-                                  int C, int R, int dims, int dtype, hipStream_t stream) {
+                                  const float* inv_freq, const int* slots, void* c_pages, void* r_pages, void* ct_pages,
+                                  int page_size, int n_tokens, int C, int R, int dims, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
-  if (C <= 0 || R <= 0 || dims < 0 || dims > R || dims % 2) return MS_BAD_ARG;
+  if (C <= 0 || R <= 0 || dims < 0 || dims > R || dims % 2 || page_size <= 0) return MS_BAD_ARG;
   dim3 grid(n_tokens), block(C >= 512 ? 256 : 128);
   if (dtype == MS_F32)
     latent_kv_store_kernel<float><<<grid, block, 0, stream>>>((const float*)kv, (size_t)kv_stride, norm_w, eps, positions, inv_freq,
-                                                              slots, (float*)c_pages, (float*)r_pages, C, R, dims);
+                                                              slots, (float*)c_pages, (float*)r_pages, (float*)ct_pages, page_size, C, R, dims);
   else if (dtype == MS_BF16)
     latent_kv_store_kernel<bf16><<<grid, block, 0, stream>>>((const bf16*)kv, (size_t)kv_stride, norm_w, eps, positions, inv_freq,
-                                                             slots, (bf16*)c_pages, (bf16*)r_pages, C, R, dims);
+                                                             slots, (bf16*)c_pages, (bf16*)r_pages, (bf16*)ct_pages, page_size, C, R, dims);
   else return MS_BAD_ARG;
   return ms_launch_status();
 }

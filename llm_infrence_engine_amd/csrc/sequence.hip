@@ -77,15 +77,16 @@ __global__ void short_conv_update_kernel(const T* __restrict__ x, size_t x_strid
 // LDS, then the chunk's tokens are walked in order.  The chunk is as long as LDS allows, up to 16 tokens.
 constexpr int DELTA_CHUNK = 16;
 
-template <typename T, int DPT>
+template <typename T, int DPT, int LPC>
 __global__ void __launch_bounds__(256)
 gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, size_t qkv_stride,
                    const float* __restrict__ a, const T* __restrict__ b, size_t b_stride,
                    const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ state,
                    const int* __restrict__ q_start, const int* __restrict__ state_slots, float* __restrict__ out,
-                   int H, int G, int D, int E, int lpc, int cols_per_block, int chunk) {
+                   int H, int G, int D, int E, int cols_per_block, int chunk) {
   extern __shared__ __align__(16) float lds[];
-  const int Dp = DPT * lpc;                 // padded key size
+  constexpr int lpc = LPC;
+  constexpr int Dp = DPT * LPC;             // padded key size
   float* qs = lds;                          // [chunk][Dp]
   float* ks = qs + chunk * Dp;
   float* gs = ks + chunk * Dp;
@@ -143,27 +144,30 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
       const float* kt = ks + t * Dp + part * DPT;
       const float* gt = gs + t * Dp + part * DPT;
       float kv = 0.f;
+      float kk[DPT];     // the token's key rows stay in registers for the write that follows the read
 #pragma unroll
       for (int ii = 0; ii < DPT; ii += 4) {
         const float4 g4 = *reinterpret_cast<const float4*>(gt + ii);
         const float4 k4 = *reinterpret_cast<const float4*>(kt + ii);
+        kk[ii] = k4.x; kk[ii + 1] = k4.y; kk[ii + 2] = k4.z; kk[ii + 3] = k4.w;
         S[ii] *= g4.x; S[ii + 1] *= g4.y; S[ii + 2] *= g4.z; S[ii + 3] *= g4.w;
         kv = fmaf(S[ii], k4.x, kv); kv = fmaf(S[ii + 1], k4.y, kv);
         kv = fmaf(S[ii + 2], k4.z, kv); kv = fmaf(S[ii + 3], k4.w, kv);
       }
-      for (int o = 1; o < lpc; o <<= 1) kv += __shfl_xor(kv, o, MS_WAVE);
+#pragma unroll
+      for (int o = 1; o < LPC; o <<= 1) kv += __shfl_xor(kv, o, MS_WAVE);
       const float u = bs[t] * (vs[t * cols_per_block + tid / lpc] - kv);
       float o_sum = 0.f;
 #pragma unroll
       for (int ii = 0; ii < DPT; ii += 4) {
-        const float4 k4 = *reinterpret_cast<const float4*>(kt + ii);
         const float4 q4 = *reinterpret_cast<const float4*>(qt + ii);
-        S[ii] = fmaf(k4.x, u, S[ii]); S[ii + 1] = fmaf(k4.y, u, S[ii + 1]);
-        S[ii + 2] = fmaf(k4.z, u, S[ii + 2]); S[ii + 3] = fmaf(k4.w, u, S[ii + 3]);
+        S[ii] = fmaf(kk[ii], u, S[ii]); S[ii + 1] = fmaf(kk[ii + 1], u, S[ii + 1]);
+        S[ii + 2] = fmaf(kk[ii + 2], u, S[ii + 2]); S[ii + 3] = fmaf(kk[ii + 3], u, S[ii + 3]);
         o_sum = fmaf(S[ii], q4.x, o_sum); o_sum = fmaf(S[ii + 1], q4.y, o_sum);
         o_sum = fmaf(S[ii + 2], q4.z, o_sum); o_sum = fmaf(S[ii + 3], q4.w, o_sum);
       }
-      for (int o = 1; o < lpc; o <<= 1) o_sum += __shfl_xor(o_sum, o, MS_WAVE);
+#pragma unroll
+      for (int o = 1; o < LPC; o <<= 1) o_sum += __shfl_xor(o_sum, o, MS_WAVE);
       if (live && part == 0) out[((size_t)(s0 + c0 + t) * H + h) * E + col] = o_sum;
     }
   }
@@ -247,13 +251,16 @@ extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long 
   if (n_requests <= 0) return MS_OK;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return MS_BAD_ARG;
   if (dim > 512 || n_requests > 65535 || heads > 65535) return MS_UNSUPPORTED;
-  // rows of a column a lane holds (DPT) and lanes a column is spread over (lpc): as few lanes as keep DPT <= 64
-  int lpc = 1;
-  while ((dim + lpc - 1) / lpc > 64) lpc *= 2;
-  // a short column leaves registers free: spread it further while the block still has a wave's worth of columns
-  while (lpc < 8 && (dim + lpc - 1) / lpc > 16 && vdim * lpc < 128) lpc *= 2;
-  const int per = (dim + lpc - 1) / lpc;
-  const int dpt = per <= 8 ? 8 : per <= 16 ? 16 : per <= 32 ? 32 : 64;
+  // lanes a column of the state is spread over (lpc) and rows each of them holds (dpt): sixteen rows a lane where the
+  // key size allows, so that a token costs a lane few dependent operations and a head's columns spread over many waves
+  int lpc, dpt;
+  if (dim <= 8) { lpc = 1; dpt = 8; }
+  else if (dim <= 16) { lpc = 1; dpt = 16; }
+  else if (dim <= 32) { lpc = 2; dpt = 16; }
+  else if (dim <= 64) { lpc = 4; dpt = 16; }
+  else if (dim <= 128) { lpc = 8; dpt = 16; }
+  else if (dim <= 256) { lpc = 8; dpt = 32; }
+  else { lpc = 8; dpt = 64; }
   int threads = vdim * lpc;
   threads = threads >= 256 ? 256 : ((threads + MS_WAVE - 1) / MS_WAVE) * MS_WAVE;
   const int cols = threads / lpc;
@@ -263,17 +270,19 @@ extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long 
   while (chunk > 1 && chunk * per_token > 65536) chunk /= 2;
   const size_t lds = chunk * per_token;
   if (lds > 65536) return MS_UNSUPPORTED;
-#define LAUNCH(T, DPT)                                                                                                  \
-  gated_delta_kernel<T, DPT><<<grid, block, lds, stream>>>((const T*)q, (const T*)k, (const T*)v, (size_t)qkv_stride, \
-                                                           a, (const T*)b, (size_t)b_stride, A_log, dt_bias, state,   \
-                                                           q_start, state_slots, out, heads, kv_heads, dim, vdim,     \
-                                                           lpc, cols, chunk)
+#define LAUNCH(T, DPT, LPC)                                                                                             \
+  gated_delta_kernel<T, DPT, LPC><<<grid, block, lds, stream>>>(                                                        \
+      (const T*)q, (const T*)k, (const T*)v, (size_t)qkv_stride, a, (const T*)b, (size_t)b_stride, A_log, dt_bias,     \
+      state, q_start, state_slots, out, heads, kv_heads, dim, vdim, cols, chunk)
 #define BY_DPT(T)                                                                                                       \
   do {                                                                                                                  \
-    if (dpt == 8) LAUNCH(T, 8);                                                                                         \
-    else if (dpt == 16) LAUNCH(T, 16);                                                                                  \
-    else if (dpt == 32) LAUNCH(T, 32);                                                                                  \
-    else LAUNCH(T, 64);                                                                                                 \
+    if (dpt == 8) LAUNCH(T, 8, 1);                                                                                      \
+    else if (dpt == 16 && lpc == 1) LAUNCH(T, 16, 1);                                                                   \
+    else if (dpt == 16 && lpc == 2) LAUNCH(T, 16, 2);                                                                   \
+    else if (dpt == 16 && lpc == 4) LAUNCH(T, 16, 4);                                                                   \
+    else if (dpt == 16) LAUNCH(T, 16, 8);                                                                               \
+    else if (dpt == 32) LAUNCH(T, 32, 8);                                                                               \
+    else LAUNCH(T, 64, 8);                                                                                              \
   } while (0)
   if (dtype == MS_F32) BY_DPT(float);
   else if (dtype == MS_BF16) BY_DPT(bf16);

@@ -83,8 +83,11 @@ _SIGNATURES = {
     "ms_rms_norm_rows": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "ms_rotary_pairs": [_c_ptr, _c_ll, _c_ll, _c_ptr, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
                         _c_ptr],
-    "ms_latent_kv_store": [_c_ptr, _c_ll, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
-                           _c_int, _c_int, _c_ptr],
+    "ms_latent_kv_store": [_c_ptr, _c_ll, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                           _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_latent_attention_mfma": [_c_ptr, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                 _c_ptr, _c_ll, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float,
+                                 _c_int, _c_ptr],
     "ms_latent_attention": [_c_ptr, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                             _c_ptr, _c_ll, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float, _c_int, _c_int,
                             _c_ptr],
@@ -987,23 +990,33 @@ def rotary_pairs(src: torch.Tensor, dst: torch.Tensor, positions: torch.Tensor, 
     return dst
 
 
+def latent_mfma_sizes(C: int, R: int) -> bool:
+    """Whether the matrix-core attention over latents has a variant for a latent of C and a rotated part of R entries
+    (the library's ms_latent_attention_mfma_supported says the same, and more about pages)."""
+    return C in (128, 256, 512) and R in (32, 64)
+
+
 def latent_kv_store(kv: torch.Tensor, norm_weight: torch.Tensor, eps: float, positions: torch.Tensor, inv_freq: torch.Tensor,
-                    slot_mapping: torch.Tensor, c_pages: torch.Tensor, r_pages: torch.Tensor) -> None:
+                    slot_mapping: torch.Tensor, c_pages: torch.Tensor, r_pages: torch.Tensor,
+                    ct_pages: Optional[torch.Tensor] = None) -> None:
     """kv [N, C + R]: the RMS norm of its first C columns (times ``norm_weight``) goes to ``c_pages`` [P, 1, page, C], its
-    last R columns, turned pair by pair, to ``r_pages`` [P, 1, page, R], at ``slot_mapping`` (< 0: not stored)."""
+    last R columns, turned pair by pair, to ``r_pages`` [P, 1, page, R], at ``slot_mapping`` (< 0: not stored).
+    ``ct_pages`` [P, 1, C, page], if given, takes the same latents transposed."""
     N = kv.shape[0]
     _check(c_pages, "c_pages", kv.dtype, (None, 1, None, None))
     C = c_pages.shape[3]
     _check(r_pages, "r_pages", kv.dtype, (c_pages.shape[0], 1, c_pages.shape[2], None))
     R = r_pages.shape[3]
+    if ct_pages is not None:
+        _check(ct_pages, "ct_pages", kv.dtype, (c_pages.shape[0], 1, C, c_pages.shape[2]))
     ks = _rows2d(kv, "kv", None, C + R)
     _check(norm_weight, "norm_weight", torch.float32, (C,))
     _check(positions, "positions", torch.int32, (N,))
     _check(slot_mapping, "slot_mapping", torch.int32, (N,))
     _check(inv_freq, "inv_freq", torch.float32)
     _call("ms_latent_kv_store", kv.data_ptr(), ks, norm_weight.data_ptr(), float(eps), positions.data_ptr(),
-          inv_freq.data_ptr(), slot_mapping.data_ptr(), c_pages.data_ptr(), r_pages.data_ptr(), N, C, R,
-          2 * inv_freq.numel(), _code(kv.dtype), _stream())
+          inv_freq.data_ptr(), slot_mapping.data_ptr(), c_pages.data_ptr(), r_pages.data_ptr(), _ptr(ct_pages),
+          c_pages.shape[2], N, C, R, 2 * inv_freq.numel(), _code(kv.dtype), _stream())
 
 
 def latent_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, scale: float, window: Optional[int] = None,
@@ -1030,6 +1043,20 @@ def latent_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, scale: float, 
         _check(kv.table_rows, "table_rows", torch.int32)
     if sink is not None:
         _check(sink, "sink", torch.float32, (H,))
+    ct_pages = kv.pages.get("ct")
+    if (q.dtype == torch.bfloat16 and ct_pages is not None and kv.transposed.get("ct") and latent_mfma_sizes(C, R)
+            and page_size % 16 == 0 and qt % 8 == 0 and qh % 8 == 0 and ot % 4 == 0 and oh % 4 == 0
+            and q.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0 and getattr(ctx, "max_q_len", 0) > 0):
+        # the matrix-core kernel: it reads the latents' transposed copy as the operand of the weighted sum
+        _check(ct_pages, "ct_pages", q.dtype, (P, 1, C, page_size))
+        Rq = ctx.num_requests
+        _check(ctx.q_start, "q_start", torch.int32, (Rq + 1,))
+        _check(ctx.context_lens, "context_lens", torch.int32, (Rq,))
+        _call("ms_latent_attention_mfma", q.data_ptr(), qt, qh, c_pages.data_ptr(), r_pages.data_ptr(), ct_pages.data_ptr(),
+              kv.block_table.data_ptr(), kv.block_table.shape[1], _ptr(kv.table_rows), ctx.q_start.data_ptr(),
+              ctx.context_lens.data_ptr(), _ptr(sink), out.data_ptr(), ot, oh, Rq, ctx.max_q_len, H, C, R, page_size, P,
+              float(scale), int(window or 0), _stream())
+        return out
     _call("ms_latent_attention", q.data_ptr(), qt, qh, c_pages.data_ptr(), r_pages.data_ptr(), kv.block_table.data_ptr(),
           kv.block_table.shape[1], _ptr(kv.table_rows), _ptr(ctx.n_live_tokens), ctx.token_req.data_ptr(),
           ctx.positions.data_ptr(), _ptr(sink), out.data_ptr(), ot, oh, N, H, C, R, page_size, P, float(scale),

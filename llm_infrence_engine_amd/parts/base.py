@@ -42,14 +42,17 @@ class PageTensor:
     """One tensor of a cache page: ``heads`` x ``width`` values per token, kept as [heads, page_size, width].
     With ``transpose_at`` = n the pool keeps it as [heads, width, page_size] instead whenever the page size is
     a multiple of n (a mixer asks for that when its kernels read the tensor as a matrix operand as it lies),
-    with ``transpose_in`` only when the cache holds that type.  What a part declares here does not depend on
-    whether it has been loaded or in which type: the pool, which knows both, decides."""
+    with ``transpose_in`` only when the cache holds that type.  ``only_transposed``: the tensor is a second copy of
+    another for kernels that want it transposed, and is left out of the pool altogether when it would not be kept
+    so.  What a part declares here does not depend on whether it has been loaded or in which type: the pool, which
+    knows both, decides."""
 
     name: str
     heads: int
     width: int
     transpose_at: Optional[int] = None
     transpose_in: Optional[torch.dtype] = None
+    only_transposed: bool = False
 
 
 @dataclass(frozen=True)

@@ -67,7 +67,13 @@ class LatentAttention(Mixer):
 
     # ---- cache: the latent and the shared rotated key part
     def cache_need(self):
-        return CacheNeed((PageTensor("c", 1, self.kv_rank), PageTensor("kr", 1, self.rot_dim)), self.window)
+        tensors = [PageTensor("c", 1, self.kv_rank), PageTensor("kr", 1, self.rot_dim)]
+        if ops.latent_mfma_sizes(self.kv_rank, self.rot_dim):
+            # the matrix-core attention weighs the latents with the keys along a row: a transposed copy, kept only in
+            # bfloat16 with pages of a multiple of 16 tokens
+            tensors.append(PageTensor("ct", 1, self.kv_rank, transpose_at=16, transpose_in=torch.bfloat16,
+                                      only_transposed=True))
+        return CacheNeed(tuple(tensors), self.window)
 
     # ---- step
     def forward(self, h, ctx, kv, state):
@@ -83,7 +89,7 @@ class LatentAttention(Mixer):
         q = linear.linear(cq, self.w_uq).view(N, H, D + R)
         if kv.store:
             ops.latent_kv_store(proj[:, kv_at:g_at], self.kv_norm, self.eps, ctx.positions, self.position.inv_freq,
-                                kv.slot_mapping, kv.pages["c"], kv.pages["kr"])
+                                kv.slot_mapping, kv.pages["c"], kv.pages["kr"], kv.pages.get("ct"))
         q_lat = self.rt.empty(N, H, C + R)
         ops.head_matmul(q[:, :, :D], self.m_uk, q_lat[:, :, :C])
         self.position.rotate(q[:, :, D:], q_lat[:, :, C:], ctx)
