@@ -37,7 +37,8 @@ __global__ void head_matmul_kernel(const T* __restrict__ in, size_t in_tok, size
 #pragma unroll
   for (int t = 0; t < HM_TOKENS; ++t) acc[t] = 0.f;
   const T* Mh = M + (size_t)h * I * J + j;
-  for (int i = 0; i < I; ++i) {
+#pragma unroll 8
+  for (int i = 0; i < I; ++i) {   // eight rows of M in flight: the loop waits for memory, not for arithmetic
     const float m = to_float(Mh[(size_t)i * J]);
     const float4 a = *reinterpret_cast<const float4*>(xs + i * HM_TOKENS);
     const float4 b = *reinterpret_cast<const float4*>(xs + i * HM_TOKENS + 4);

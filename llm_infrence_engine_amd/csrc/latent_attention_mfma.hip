@@ -2,7 +2,9 @@
 //
 // All query heads read the same keys [c_j ; kr_j] and the same values c_j, so a *column* is a (token, head) pair
 // and a wave owns 16 consecutive columns of one request (head running fastest): every key it loads serves 16
-// heads, or several tokens' heads.  Keys are walked in blocks of 32:
+// heads, or several tokens' heads.  The waves of a block share one tile of 16 columns and take its key blocks in turn,
+// each with its own running maximum, sum and accumulators, merged through LDS at the end in wave order: a single
+// decoded token's keys are then walked by four waves at once.  Keys are walked in blocks of 32:
 //
 //   S^T[key, col]  = K[key, :] . Q^T[:, col]      A operand: 16 keys x 32 entries read in place from the pages (the
 //                                                 latent's C entries, then the rotated part's R), B: the query
@@ -13,8 +15,8 @@
 //
 // The sums of the exponentials come from one more product with ones (the bfloat16 values that weigh the latents).
 // Values past the last visible key are zeroed before use and pages past the context are never dereferenced.
-// Launch: grid (column tiles of the longest portion / WAVES, requests); a wave without a tile leaves at once, so
-// the launch depends on the step's number of requests and longest portion only.
+// Launch: grid (column tiles of the longest portion, requests); a block without a tile leaves at once, so the launch
+// depends on the step's number of requests and longest portion only.
 #include "common.h"
 #include "api.h"
 
@@ -35,6 +37,8 @@ latent_attention_mfma_kernel(const bf16* __restrict__ q, size_t q_tok, size_t q_
                              const float* __restrict__ sink, bf16* __restrict__ out, size_t out_tok, size_t out_head,
                              int H, int page_size, float scale_log2e, int window) {
   constexpr int KS_C = C / 32, KS_R = R / 32, CT = C / 16;
+  __shared__ float sm_m[LM_WAVES][16], sm_l[LM_WAVES][16];
+  __shared__ f32x4 sm_o[CT][MS_WAVE];
   const int lane = threadIdx.x & (MS_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MS_WAVE);
   const int col16 = lane & 15, kq = lane >> 4;
@@ -42,8 +46,8 @@ latent_attention_mfma_kernel(const bf16* __restrict__ q, size_t q_tok, size_t q_
   const int q0 = q_start[r];
   const int qlen = q_start[r + 1] - q0;
   const int ncols = qlen * H;
-  const int c0 = (blockIdx.x * LM_WAVES + wave) * 16;
-  if (c0 >= ncols) return;                         // the whole wave; there is no block-wide barrier below
+  const int c0 = blockIdx.x * 16;
+  if (c0 >= ncols) return;                         // the whole block
   const int start_pos = context_lens[r] - qlen;
   const int* table = block_table + (size_t)(table_rows ? table_rows[r] : r) * table_stride;
 
@@ -72,7 +76,7 @@ latent_attention_mfma_kernel(const bf16* __restrict__ q, size_t q_tok, size_t q_
 #pragma unroll
   for (int t = 0; t < CT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int base = (key_lo / 32) * 32; base <= key_hi; base += 32) {
+  for (int base = (key_lo / 32 + wave) * 32; base <= key_hi; base += 32 * LM_WAVES) {
     // the two 16-key halves of the block: a half lies in one page (pages hold a multiple of 16 keys)
     size_t row0[2];     // first key's row in the pools (page * page_size + offset); the null page past the context
 #pragma unroll
@@ -147,8 +151,36 @@ latent_attention_mfma_kernel(const bf16* __restrict__ q, size_t q_tok, size_t q_
       o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, p, o[t], 0, 0, 0);
     }
   }
-  if (pos < 0) return;
   float l = lsum[0];      // every row of the product with ones is the column's sum
+  // merge the waves' shares (each relative to its own maximum) into wave 0, in wave order
+  if (kq == 0) { sm_m[wave][col16] = m; sm_l[wave][col16] = l; }
+  __syncthreads();
+  {
+    float big = sm_m[0][col16];
+#pragma unroll
+    for (int w = 1; w < LM_WAVES; ++w) big = fmaxf(big, sm_m[w][col16]);
+    const float safe = big == -INFINITY ? 0.f : big;
+    const float f = __builtin_amdgcn_exp2f(m - safe);      // a wave that saw no key: 0
+#pragma unroll
+    for (int t = 0; t < CT; ++t) o[t] *= f;
+    l = 0.f;
+#pragma unroll
+    for (int w = 0; w < LM_WAVES; ++w) l += sm_l[w][col16] * __builtin_amdgcn_exp2f(sm_m[w][col16] - safe);
+    m = big;
+  }
+  for (int w = 1; w < LM_WAVES; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int t = 0; t < CT; ++t) sm_o[t][lane] = o[t];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int t = 0; t < CT; ++t) o[t] += sm_o[t][lane];
+    }
+    __syncthreads();
+  }
+  if (wave != 0 || pos < 0) return;
   if (sink) {             // the sink: one more term exp(sink) in the denominator, unscaled, with no value
     const float sk = sink[head] * 1.4426950408889634f;
     const float big = fmaxf(m, sk);
@@ -190,7 +222,7 @@ extern "C" int ms_latent_attention_mfma(const void* q, long long q_tok, long lon
   if (q_tok % 8 || q_head % 8 || out_tok % 4 || out_head % 4) return MS_UNSUPPORTED;
   if (num_pages * page_size >= (1ll << 31) || n_requests > 65535) return MS_UNSUPPORTED;
   const long long tiles = ((long long)max_q_len * heads + 15) / 16;
-  dim3 grid((unsigned)((tiles + LM_WAVES - 1) / LM_WAVES), n_requests), block(LM_WAVES * MS_WAVE);
+  dim3 grid((unsigned)tiles, n_requests), block(LM_WAVES * MS_WAVE);
   const float sl = scale * 1.4426950408889634f;
 #define LAUNCH(CC, RR)                                                                                                  \
   latent_attention_mfma_kernel<CC, RR><<<grid, block, 0, stream>>>(                                                     \

@@ -67,6 +67,20 @@ __global__ void short_conv_update_kernel(const T* __restrict__ x, size_t x_strid
     if (i < hist) st[(size_t)i * C + c] = keep[i];
 }
 
+// Sum over groups of LPC neighbouring lanes (LPC a power of two up to 16, groups aligned), every lane of a group
+// getting the sum, by lane permutations inside the vector unit: within a quad lane ^ 1 and lane ^ 2, then the two
+// quads of eight lanes mirrored onto each other (all lanes of a quad hold the same value by then).
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int LPC> __device__ __forceinline__ float group_sum(float v) {
+  if (LPC >= 2) v += dpp_move<0xB1>(v);     // quad_perm [1, 0, 3, 2]
+  if (LPC >= 4) v += dpp_move<0x4E>(v);     // quad_perm [2, 3, 0, 1]
+  if (LPC >= 8) v += dpp_move<0x141>(v);    // row_half_mirror: lane i of eight <- lane 7 - i
+  if (LPC >= 16) v += dpp_move<0x140>(v);   // row_mirror: lane i of sixteen <- lane 15 - i
+  return v;
+}
+
 // ------------------------------------------------------------------------------------------------
 // The gated delta rule.  Per request and head, S [D, E] float, token by token:
 //   S <- g * S (row i by g_i);  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
@@ -109,65 +123,117 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
   const float rate = expf(A_log[h]);
   const float q_scale = 1.0f / sqrtf((float)D);
 
-  for (int c0 = 0; c0 < L; c0 += chunk) {
+  // Staging.  LT lanes share a token (the host makes the chunk no longer than the block has such groups): a lane
+  // asks for all its entries of q, k, the decay's input, and its values of v at once, a chunk ahead, so that one trip
+  // to memory serves a whole chunk and is over by the time the chunk before has been walked.
+  constexpr int LT = Dp > 256 ? 64 : 16, EPL = (Dp + LT - 1) / LT, VPL = 16;   // a whole wave to a token of the longest keys
+  const int tl = tid / LT, l16 = tid % LT;
+  float qf[EPL], kf[EPL], af[EPL], vf[VPL], bf = 0.f;
+  auto ask = [&](int c0) __attribute__((always_inline)) {
     const int cn = min(chunk, L - c0);
-    __syncthreads();   // the chunk before is done with the staging area
-    for (int t = wave; t < cn; t += nwaves) {        // a wave normalises a token's q and k
-      const size_t n = (size_t)(s0 + c0 + t);
+    if (tl < cn) {
+      const size_t n = (size_t)(s0 + c0 + tl);
       const T* qp = q + n * qkv_stride + (size_t)kvh * D;
       const T* kp = k + n * qkv_stride + (size_t)kvh * D;
-      float sq = 0.f, sk = 0.f;
-      for (int i = lane; i < D; i += MS_WAVE) {
-        const float a0 = to_float(qp[i]), a1 = to_float(kp[i]);
-        sq = fmaf(a0, a0, sq);
-        sk = fmaf(a1, a1, sk);
-      }
-      sq = wave_sum(sq);
-      sk = wave_sum(sk);
-      const float iq = q_scale / sqrtf(sq + 1e-6f), ik = 1.0f / sqrtf(sk + 1e-6f);
       const float* ap = a + n * (size_t)H * D + (size_t)h * D;
-      for (int i = lane; i < Dp; i += MS_WAVE) {
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        const int i = l16 + e * LT;
         const bool in = i < D;
-        qs[t * Dp + i] = in ? to_float(qp[i]) * iq : 0.f;
-        ks[t * Dp + i] = in ? to_float(kp[i]) * ik : 0.f;
-        gs[t * Dp + i] = in ? expf(-rate * softplus_f(ap[i] + dt_bias[(size_t)h * D + i])) : 1.f;
+        qf[e] = in ? to_float(qp[i]) : 0.f;
+        kf[e] = in ? to_float(kp[i]) : 0.f;
+        af[e] = in ? ap[i] + dt_bias[(size_t)h * D + i] : 0.f;
       }
-      if (lane == 0) bs[t] = sigmoid_f(to_float(b[n * b_stride + h]));
+      if (l16 == 0) bf = to_float(b[n * b_stride + h]);
     }
-    for (int e = tid; e < cn * cols_per_block; e += blockDim.x) {
-      const int t = e / cols_per_block, j = e - t * cols_per_block;
-      vs[e] = col0 + j < E ? to_float(v[(size_t)(s0 + c0 + t) * qkv_stride + (size_t)h * E + col0 + j]) : 0.f;
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      const int e = tid + j * blockDim.x;
+      if (e < cn * cols_per_block) {
+        const int t = e / cols_per_block, jj = e - t * cols_per_block;
+        vf[j] = col0 + jj < E ? to_float(v[(size_t)(s0 + c0 + t) * qkv_stride + (size_t)h * E + col0 + jj]) : 0.f;
+      }
+    }
+  };
+  constexpr bool ASK_AHEAD = DPT <= 32;   // the longest columns leave no registers to hold a chunk through the walk
+  if (ASK_AHEAD) ask(0);
+  for (int c0 = 0; c0 < L; c0 += chunk) {
+    const int cn = min(chunk, L - c0);
+    if (!ASK_AHEAD) ask(c0);
+    __syncthreads();   // the chunk before is done with the staging area
+    if (tl < cn) {
+      float sq = 0.f, sk = 0.f;
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) { sq = fmaf(qf[e], qf[e], sq); sk = fmaf(kf[e], kf[e], sk); }
+      sq = LT == 64 ? wave_sum(sq) : group_sum<16>(sq);
+      sk = LT == 64 ? wave_sum(sk) : group_sum<16>(sk);
+      const float iq = q_scale / sqrtf(sq + 1e-6f), ik = 1.0f / sqrtf(sk + 1e-6f);
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        const int i = l16 + e * LT;
+        if (i < Dp) {
+          const bool in = i < D;
+          qs[tl * Dp + i] = qf[e] * iq;
+          ks[tl * Dp + i] = kf[e] * ik;
+          gs[tl * Dp + i] = in ? expf(-rate * softplus_f(af[e])) : 1.f;
+        }
+      }
+      if (l16 == 0) bs[tl] = sigmoid_f(bf);
+    }
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      const int e = tid + j * blockDim.x;
+      if (e < cn * cols_per_block) vs[e] = vf[j];
     }
     __syncthreads();
-    for (int t = 0; t < cn; ++t) {
+    if (ASK_AHEAD && c0 + chunk < L) ask(c0 + chunk);
+    // the rows of the next token's q, k and g are fetched from LDS while the current token is worked on; the two
+    // sums over a column run as four chains each
+    float gn[DPT], kn[DPT], qn[DPT];
+    auto fetch = [&](int t) __attribute__((always_inline)) {
       const float* qt = qs + t * Dp + part * DPT;
       const float* kt = ks + t * Dp + part * DPT;
       const float* gt = gs + t * Dp + part * DPT;
-      float kv = 0.f;
-      float kk[DPT];     // the token's key rows stay in registers for the write that follows the read
 #pragma unroll
       for (int ii = 0; ii < DPT; ii += 4) {
         const float4 g4 = *reinterpret_cast<const float4*>(gt + ii);
         const float4 k4 = *reinterpret_cast<const float4*>(kt + ii);
-        kk[ii] = k4.x; kk[ii + 1] = k4.y; kk[ii + 2] = k4.z; kk[ii + 3] = k4.w;
-        S[ii] *= g4.x; S[ii + 1] *= g4.y; S[ii + 2] *= g4.z; S[ii + 3] *= g4.w;
-        kv = fmaf(S[ii], k4.x, kv); kv = fmaf(S[ii + 1], k4.y, kv);
-        kv = fmaf(S[ii + 2], k4.z, kv); kv = fmaf(S[ii + 3], k4.w, kv);
+        const float4 q4 = *reinterpret_cast<const float4*>(qt + ii);
+        gn[ii] = g4.x; gn[ii + 1] = g4.y; gn[ii + 2] = g4.z; gn[ii + 3] = g4.w;
+        kn[ii] = k4.x; kn[ii + 1] = k4.y; kn[ii + 2] = k4.z; kn[ii + 3] = k4.w;
+        qn[ii] = q4.x; qn[ii + 1] = q4.y; qn[ii + 2] = q4.z; qn[ii + 3] = q4.w;
       }
+    };
+    constexpr bool AHEAD = DPT <= 32;    // the longest columns leave no registers for a second set of rows
+    if (AHEAD) fetch(0);
+    for (int t = 0; t < cn; ++t) {
+      if (!AHEAD) fetch(t);
+      float gg[DPT], kk[DPT], qq[DPT];
 #pragma unroll
-      for (int o = 1; o < LPC; o <<= 1) kv += __shfl_xor(kv, o, MS_WAVE);
-      const float u = bs[t] * (vs[t * cols_per_block + tid / lpc] - kv);
-      float o_sum = 0.f;
+      for (int ii = 0; ii < DPT; ++ii) { gg[ii] = gn[ii]; kk[ii] = kn[ii]; qq[ii] = qn[ii]; }
+      const float beta_t = bs[t], v_t = vs[t * cols_per_block + tid / lpc];
+      if (AHEAD && t + 1 < cn) fetch(t + 1);
+      float kv4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ii = 0; ii < DPT; ii += 4) {
-        const float4 q4 = *reinterpret_cast<const float4*>(qt + ii);
-        S[ii] = fmaf(kk[ii], u, S[ii]); S[ii + 1] = fmaf(kk[ii + 1], u, S[ii + 1]);
-        S[ii + 2] = fmaf(kk[ii + 2], u, S[ii + 2]); S[ii + 3] = fmaf(kk[ii + 3], u, S[ii + 3]);
-        o_sum = fmaf(S[ii], q4.x, o_sum); o_sum = fmaf(S[ii + 1], q4.y, o_sum);
-        o_sum = fmaf(S[ii + 2], q4.z, o_sum); o_sum = fmaf(S[ii + 3], q4.w, o_sum);
-      }
 #pragma unroll
-      for (int o = 1; o < LPC; o <<= 1) o_sum += __shfl_xor(o_sum, o, MS_WAVE);
+        for (int j = 0; j < 4; ++j) {
+          S[ii + j] *= gg[ii + j];
+          kv4[j] = fmaf(S[ii + j], kk[ii + j], kv4[j]);
+        }
+      }
+      const float kv = group_sum<LPC>((kv4[0] + kv4[1]) + (kv4[2] + kv4[3]));
+      const float u = beta_t * (v_t - kv);
+      float o4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ii = 0; ii < DPT; ii += 4) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          S[ii + j] = fmaf(kk[ii + j], u, S[ii + j]);
+          o4[j] = fmaf(S[ii + j], qq[ii + j], o4[j]);
+        }
+      }
+      const float o_sum = group_sum<LPC>((o4[0] + o4[1]) + (o4[2] + o4[3]));
       if (live && part == 0) out[((size_t)(s0 + c0 + t) * H + h) * E + col] = o_sum;
     }
   }
@@ -265,7 +331,8 @@ extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long 
   threads = threads >= 256 ? 256 : ((threads + MS_WAVE - 1) / MS_WAVE) * MS_WAVE;
   const int cols = threads / lpc;
   dim3 grid((vdim + cols - 1) / cols, heads, n_requests), block(threads);
-  int chunk = DELTA_CHUNK;
+  const int stagers = dpt * lpc > 256 ? 64 : 16;    // lanes that stage a token
+  int chunk = DELTA_CHUNK < threads / stagers ? DELTA_CHUNK : threads / stagers;
   const size_t per_token = (3 * (size_t)dpt * lpc + cols + 1) * sizeof(float);
   while (chunk > 1 && chunk * per_token > 65536) chunk /= 2;
   const size_t lds = chunk * per_token;

@@ -990,6 +990,9 @@ def rotary_pairs(src: torch.Tensor, dst: torch.Tensor, positions: torch.Tensor, 
     return dst
 
 
+launches = {}     # how often a dispatcher below chose a kernel that tests want to see chosen: name -> times
+
+
 def latent_mfma_sizes(C: int, R: int) -> bool:
     """Whether the matrix-core attention over latents has a variant for a latent of C and a rotated part of R entries
     (the library's ms_latent_attention_mfma_supported says the same, and more about pages)."""
@@ -1048,6 +1051,7 @@ def latent_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, scale: float, 
             and page_size % 16 == 0 and qt % 8 == 0 and qh % 8 == 0 and ot % 4 == 0 and oh % 4 == 0
             and q.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0 and getattr(ctx, "max_q_len", 0) > 0):
         # the matrix-core kernel: it reads the latents' transposed copy as the operand of the weighted sum
+        launches["latent_attention_mfma"] = launches.get("latent_attention_mfma", 0) + 1
         _check(ct_pages, "ct_pages", q.dtype, (P, 1, C, page_size))
         Rq = ctx.num_requests
         _check(ctx.q_start, "q_start", torch.int32, (Rq + 1,))

@@ -476,6 +476,7 @@ def test_latent_attention_window_edges_sink_and_pages(dtype, C, R, page, window)
 
     tol = 3e-5 if dtype == torch.float32 else 5e-2
     # one step: a portion of request 0 (tokens 40..69) beside the last token of request 1
+    before = ops.launches.get("latent_attention_mfma", 0)
     toks = [(0, t) for t in range(40, 70)] + [(1, 32)]
     q = (0.5 * torch.randn(len(toks), H, C + R)).to(dtype)
     q[:, 0, 0] = 8.0 * 0.3 / scale                                       # head 0 listens for the loud feature
@@ -498,6 +499,7 @@ def test_latent_attention_window_edges_sink_and_pages(dtype, C, R, page, window)
         o = ops.latent_attention(q1.cuda(), kv, _Ctx([1], [0], starts=[t]), torch.empty(1, H, C, dtype=dtype, device="cuda"),
                                  scale, window, sink.cuda())
         assert (o[0].cpu().double() - plain(0, t, q1[0])).abs().max() < tol, t
+    assert (ops.launches.get("latent_attention_mfma", 0) > before) == (matrix_cores and dtype == torch.bfloat16)
     # without a sink the weights sum to one
     ones = ops.latent_attention(q.cuda(), kv, ctx, torch.empty(len(toks), H, C, dtype=dtype, device="cuda"), scale, window, None)
     assert torch.isfinite(ones).all()
@@ -570,7 +572,12 @@ def test_replay_against_plain(shape, tmp_path, dtype, mode):
         max_tokens = max(up(len(t)) for t in reqs.values())
         steps = {"whole": traces.whole, "bulk_then_single": lambda r: traces.bulk_then_single(r, tail=45),
                  "changing_portions": traces.changing_portions}[mode](reqs)
+    from llm_infrence_engine_amd.kernels import ops
+
+    before = ops.launches.get("latent_attention_mfma", 0)
     runner = _replay(folder, dtype, steps, tmp_path / "out", max_tokens, page)
+    if mode == "whole":      # launched kernel by kernel or captured, the shape S's attention is the matrix cores' in bfloat16
+        assert (ops.launches.get("latent_attention_mfma", 0) > before) == (name == "S" and dtype == "bfloat16")
     _compare(traces.collect(steps, tmp_path / "out", cfg["vocab"]), want, noise, dtype)
     if mode == "mixed":
         for g in runner.manager.groups:
