@@ -157,11 +157,12 @@ int ms_short_conv(const void* x, long long x_stride, const float* w, void* state
 
 // Gated delta rule with a decay per head and key channel.  q, k [n, kv_heads * dim], v [n, heads * vdim], b [n, heads]
 // in `dtype` (rows qkv_stride / b_stride apart); a float [n, heads * dim] (the decay's input before dt_bias);
-// state float [slots, heads, dim, vdim]; out float [n, heads * vdim].
+// state float [slots, heads, dim, vdim]; out float [n, heads * vdim].  single_tokens: the caller knows that no request
+// has more than one token (a decode step).
 int ms_gated_delta(const void* q, const void* k, const void* v, long long qkv_stride, const float* a, const void* b,
                    long long b_stride, const float* A_log, const float* dt_bias, float* state, const int* q_start,
                    const int* state_slots, float* out, int n_requests, int heads, int kv_heads, int dim, int vdim,
-                   int dtype, hipStream_t stream);
+                   int single_tokens, int dtype, hipStream_t stream);
 
 // out[n, h, :] = o[n, h, :] / rms(o[n, h, :]) * weight * sigmoid(gate[n, h, :]); o float, gate and out in `dtype`.
 int ms_gated_head_norm(const float* o, const float* weight, const void* gate, long long gate_stride, void* out,

@@ -91,8 +91,10 @@ template <int LPC> __device__ __forceinline__ float group_sum(float v) {
 // LDS, then the chunk's tokens are walked in order.  The chunk is as long as LDS allows, up to 16 tokens.
 constexpr int DELTA_CHUNK = 16;
 
-template <typename T, int DPT, int LPC>
-__global__ void __launch_bounds__(256)
+// SINGLE: every request of the step has one token (a decode step).  Nothing is asked or fetched ahead then, which
+// leaves registers for three blocks to a CU: the step is the read and the write of the states, and needs them in flight.
+template <typename T, int DPT, int LPC, bool SINGLE>
+__global__ void __launch_bounds__(256, SINGLE ? 3 : 1)
 gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, size_t qkv_stride,
                    const float* __restrict__ a, const T* __restrict__ b, size_t b_stride,
                    const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ state,
@@ -126,7 +128,7 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
   // Staging.  LT lanes share a token (the host makes the chunk no longer than the block has such groups): a lane
   // asks for all its entries of q, k, the decay's input, and its values of v at once, a chunk ahead, so that one trip
   // to memory serves a whole chunk and is over by the time the chunk before has been walked.
-  constexpr int LT = Dp > 256 ? 64 : 16, EPL = (Dp + LT - 1) / LT, VPL = 16;   // a whole wave to a token of the longest keys
+  constexpr int LT = Dp > 256 ? 64 : 16, EPL = (Dp + LT - 1) / LT, VPL = SINGLE ? 1 : 16 / LPC;   // a chunk has at most 16 / LPC values of v a lane   // a whole wave to a token of the longest keys
   const int tl = tid / LT, l16 = tid % LT;
   float qf[EPL], kf[EPL], af[EPL], vf[VPL], bf = 0.f;
   auto ask = [&](int c0) __attribute__((always_inline)) {
@@ -155,7 +157,7 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
       }
     }
   };
-  constexpr bool ASK_AHEAD = DPT <= 32;   // the longest columns leave no registers to hold a chunk through the walk
+  constexpr bool ASK_AHEAD = DPT <= 32 && !SINGLE;   // the longest columns leave no registers to hold a chunk through the walk
   if (ASK_AHEAD) ask(0);
   for (int c0 = 0; c0 < L; c0 += chunk) {
     const int cn = min(chunk, L - c0);
@@ -204,7 +206,7 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
         qn[ii] = q4.x; qn[ii + 1] = q4.y; qn[ii + 2] = q4.z; qn[ii + 3] = q4.w;
       }
     };
-    constexpr bool AHEAD = DPT <= 32;    // the longest columns leave no registers for a second set of rows
+    constexpr bool AHEAD = DPT <= 32 && !SINGLE;    // the longest columns leave no registers for a second set of rows
     if (AHEAD) fetch(0);
     for (int t = 0; t < cn; ++t) {
       if (!AHEAD) fetch(t);
@@ -313,7 +315,8 @@ extern "C" int ms_short_conv(const void* x, long long x_stride, const float* w, 
 extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long long qkv_stride, const float* a,
                               const void* b, long long b_stride, const float* A_log, const float* dt_bias,
                               float* state, const int* q_start, const int* state_slots, float* out, int n_requests,
-                              int heads, int kv_heads, int dim, int vdim, int dtype, hipStream_t stream) {
+                              int heads, int kv_heads, int dim, int vdim, int single_tokens, int dtype,
+                              hipStream_t stream) {
   if (n_requests <= 0) return MS_OK;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return MS_BAD_ARG;
   if (dim > 512 || n_requests > 65535 || heads > 65535) return MS_UNSUPPORTED;
@@ -337,10 +340,15 @@ extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long 
   while (chunk > 1 && chunk * per_token > 65536) chunk /= 2;
   const size_t lds = chunk * per_token;
   if (lds > 65536) return MS_UNSUPPORTED;
-#define LAUNCH(T, DPT, LPC)                                                                                             \
-  gated_delta_kernel<T, DPT, LPC><<<grid, block, lds, stream>>>(                                                        \
+#define LAUNCH1(T, DPT, LPC, ONE)                                                                                       \
+  gated_delta_kernel<T, DPT, LPC, ONE><<<grid, block, lds, stream>>>(                                                   \
       (const T*)q, (const T*)k, (const T*)v, (size_t)qkv_stride, a, (const T*)b, (size_t)b_stride, A_log, dt_bias,     \
       state, q_start, state_slots, out, heads, kv_heads, dim, vdim, cols, chunk)
+#define LAUNCH(T, DPT, LPC)                                                                                             \
+  do {                                                                                                                  \
+    if (single_tokens && DPT <= 16) LAUNCH1(T, DPT, LPC, (DPT <= 16));                                                       \
+    else LAUNCH1(T, DPT, LPC, false);                                                                                   \
+  } while (0)
 #define BY_DPT(T)                                                                                                       \
   do {                                                                                                                  \
     if (dpt == 8) LAUNCH(T, 8, 1);                                                                                      \
@@ -356,6 +364,7 @@ extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long 
   else return MS_BAD_ARG;
 #undef BY_DPT
 #undef LAUNCH
+#undef LAUNCH1
   return ms_launch_status();
 }
 

@@ -75,7 +75,7 @@ _SIGNATURES = {
     "ms_short_conv": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int,
                       _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gated_delta": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gated_head_norm": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "ms_xielu": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_head_matmul": [_c_ptr, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_ll, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int,
@@ -908,7 +908,7 @@ def gated_delta(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tens
         raise ValueError(f"{heads} heads cannot share {kv_heads} query/key heads")
     _call("ms_gated_delta", q.data_ptr(), k.data_ptr(), v.data_ptr(), sq, a.data_ptr(), b.data_ptr(), sb, A_log.data_ptr(),
           dt_bias.data_ptr(), state.data_ptr(), ctx.q_start.data_ptr(), ctx.state_slots.data_ptr(), out.data_ptr(), R,
-          heads, kv_heads, dim, vdim, _code(q.dtype), _stream())
+          heads, kv_heads, dim, vdim, int(getattr(ctx, "max_q_len", 0) == 1), _code(q.dtype), _stream())
     return out
 
 
