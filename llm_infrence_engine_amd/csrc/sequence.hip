@@ -189,10 +189,10 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
     }
     __syncthreads();
     if (ASK_AHEAD && c0 + chunk < L) ask(c0 + chunk);
-    // the rows of the next token's q, k and g are fetched from LDS while the current token is worked on; the two
-    // sums over a column run as four chains each
-    float gn[DPT], kn[DPT], qn[DPT];
-    auto fetch = [&](int t) __attribute__((always_inline)) {
+    // the rows of the next token's q, k and g are fetched from LDS while the current token is worked on (two sets of
+    // registers taken in turn, so that nothing is copied); the two sums over a column run as four chains each
+    struct Rows { float g[DPT], k[DPT], q[DPT]; };
+    auto fetch = [&](Rows& r, int t) __attribute__((always_inline)) {
       const float* qt = qs + t * Dp + part * DPT;
       const float* kt = ks + t * Dp + part * DPT;
       const float* gt = gs + t * Dp + part * DPT;
@@ -201,27 +201,19 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
         const float4 g4 = *reinterpret_cast<const float4*>(gt + ii);
         const float4 k4 = *reinterpret_cast<const float4*>(kt + ii);
         const float4 q4 = *reinterpret_cast<const float4*>(qt + ii);
-        gn[ii] = g4.x; gn[ii + 1] = g4.y; gn[ii + 2] = g4.z; gn[ii + 3] = g4.w;
-        kn[ii] = k4.x; kn[ii + 1] = k4.y; kn[ii + 2] = k4.z; kn[ii + 3] = k4.w;
-        qn[ii] = q4.x; qn[ii + 1] = q4.y; qn[ii + 2] = q4.z; qn[ii + 3] = q4.w;
+        r.g[ii] = g4.x; r.g[ii + 1] = g4.y; r.g[ii + 2] = g4.z; r.g[ii + 3] = g4.w;
+        r.k[ii] = k4.x; r.k[ii + 1] = k4.y; r.k[ii + 2] = k4.z; r.k[ii + 3] = k4.w;
+        r.q[ii] = q4.x; r.q[ii + 1] = q4.y; r.q[ii + 2] = q4.z; r.q[ii + 3] = q4.w;
       }
     };
-    constexpr bool AHEAD = DPT <= 32 && !SINGLE;    // the longest columns leave no registers for a second set of rows
-    if (AHEAD) fetch(0);
-    for (int t = 0; t < cn; ++t) {
-      if (!AHEAD) fetch(t);
-      float gg[DPT], kk[DPT], qq[DPT];
-#pragma unroll
-      for (int ii = 0; ii < DPT; ++ii) { gg[ii] = gn[ii]; kk[ii] = kn[ii]; qq[ii] = qn[ii]; }
-      const float beta_t = bs[t], v_t = vs[t * cols_per_block + tid / lpc];
-      if (AHEAD && t + 1 < cn) fetch(t + 1);
+    auto token = [&](const Rows& r, int t, float beta_t, float v_t) __attribute__((always_inline)) {
       float kv4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ii = 0; ii < DPT; ii += 4) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          S[ii + j] *= gg[ii + j];
-          kv4[j] = fmaf(S[ii + j], kk[ii + j], kv4[j]);
+          S[ii + j] *= r.g[ii + j];
+          kv4[j] = fmaf(S[ii + j], r.k[ii + j], kv4[j]);
         }
       }
       const float kv = group_sum<LPC>((kv4[0] + kv4[1]) + (kv4[2] + kv4[3]));
@@ -231,12 +223,35 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
       for (int ii = 0; ii < DPT; ii += 4) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          S[ii + j] = fmaf(kk[ii + j], u, S[ii + j]);
-          o4[j] = fmaf(S[ii + j], qq[ii + j], o4[j]);
+          S[ii + j] = fmaf(r.k[ii + j], u, S[ii + j]);
+          o4[j] = fmaf(S[ii + j], r.q[ii + j], o4[j]);
         }
       }
       const float o_sum = group_sum<LPC>((o4[0] + o4[1]) + (o4[2] + o4[3]));
       if (live && part == 0) out[((size_t)(s0 + c0 + t) * H + h) * E + col] = o_sum;
+    };
+    constexpr bool AHEAD = DPT <= 32 && !SINGLE;    // the longest columns leave no registers for a second set of rows
+    const int my_col = tid / lpc;
+    if (AHEAD) {
+      Rows ra, rb;
+      fetch(ra, 0);
+      for (int t = 0; t < cn; t += 2) {
+        const float b0 = bs[t], v0 = vs[t * cols_per_block + my_col];
+        const bool two = t + 1 < cn;
+        if (two) fetch(rb, t + 1);
+        token(ra, t, b0, v0);
+        if (two) {
+          const float b1 = bs[t + 1], v1 = vs[(t + 1) * cols_per_block + my_col];
+          if (t + 2 < cn) fetch(ra, t + 2);
+          token(rb, t + 1, b1, v1);
+        }
+      }
+    } else {
+      Rows ra;
+      for (int t = 0; t < cn; ++t) {
+        fetch(ra, t);
+        token(ra, t, bs[t], vs[t * cols_per_block + my_col]);
+      }
     }
   }
 #pragma unroll

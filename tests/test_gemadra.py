@@ -649,6 +649,13 @@ def test_greedy_generation_through_the_engine(shape, dtype):
     m = llm.engine.runner.manager
     m.check_invariants()
     assert all(g.allocator.num_in_use() == 0 for g in m.groups) and m.num_requests() == 0
+    if dtype == "bfloat16":
+        # four decode steps to a graph launch, each fed the token the one before chose on the device: the same tokens
+        del llm
+        several = eng.LLM(str(folder), dtype=dtype, block_size=PAGES[name], max_len=128, max_seqs=3, max_prefill_chunk=7,
+                          decode_steps_per_launch=4)
+        again = several.generate(prompts, eng.SamplingParams(max_new_tokens=12))
+        assert [o.token_ids for o in again] == [o.token_ids for o in outs]
 
 
 @gpu
