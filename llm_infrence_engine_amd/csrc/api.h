@@ -12,6 +12,10 @@ int ms_rms_norm(float* x, const void* delta, int delta_dtype, int n_partials, lo
                 const float* weight, const int* rows, void* out, int n_rows, int hidden, float eps, int write_back,
                 int dtype, hipStream_t stream);
 
+// the same rows normalised once and scaled twice: out1 = w1 * n(x (+ delta)), out2 = w2 * n(x (+ delta)); the sum is kept in x
+int ms_rms_norm_pair(float* x, const void* delta, int delta_dtype, const float* w1, const float* w2, void* out1, void* out2,
+                     int n_rows, int hidden, float eps, int dtype, hipStream_t stream);
+
 int ms_bias_add(void* x, const float* bias, int n_rows, int width, int dtype, hipStream_t stream);
 
 // tables / slots: host arrays of n_groups device pointers (block table int32 [table rows, table_stride], slot
@@ -149,11 +153,12 @@ int ms_sample(const float* logits, long long ld, int n_rows, int vocab, const fl
 // slot state_slots[r]; token_req [n_tokens]; n_live_tokens (may be null): tokens from there on belong to no request.
 // Short causal convolution per channel: w float [channels, taps] (last column: the current token), state
 // [slots, taps - 1, channels] in `dtype`.  mode 0: the sum, 1: x + the sum, 2: silu(the sum).  out must not be x.
-// With update_state the state becomes the last taps - 1 inputs of every request that has tokens.
+// With update_state the state becomes the last taps - 1 inputs of every request that has tokens (single_tokens: the
+// caller knows that no request has more than one token, and the same kernel moves the state on).
 int ms_short_conv(const void* x, long long x_stride, const float* w, void* state, const int* token_req,
                   const int* q_start, const int* state_slots, const int* n_live_tokens, void* out, long long out_stride,
-                  int n_tokens, int n_requests, int channels, int taps, int mode, int update_state, int dtype,
-                  hipStream_t stream);
+                  int n_tokens, int n_requests, int channels, int taps, int mode, int update_state, int single_tokens,
+                  int dtype, hipStream_t stream);
 
 // Gated delta rule with a decay per head and key channel.  q, k [n, kv_heads * dim], v [n, heads * vdim], b [n, heads]
 // in `dtype` (rows qkv_stride / b_stride apart); a float [n, heads * dim] (the decay's input before dt_bias);

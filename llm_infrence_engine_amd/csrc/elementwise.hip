@@ -114,6 +114,50 @@ extern "C" int ms_rms_norm(float* x, const void* delta, int delta_dtype, int n_p
 }
 
 // ------------------------------------------------------------------------------------------------
+// Two norms of the same rows with two scales (a layer whose branches both read x): the sum x += delta, the sum of
+// squares and the normalisation happen once.  out1 = w1 * n(x), out2 = w2 * n(x).
+template <typename T, typename TD>
+__global__ void rms_norm_pair_kernel(float* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ w1,
+                                     const float* __restrict__ w2, T* __restrict__ out1, T* __restrict__ out2, int H,
+                                     float eps) {
+  __shared__ float red[16];
+  float* xr = x + (size_t)blockIdx.x * H;
+  const TD* dr = delta ? delta + (size_t)blockIdx.x * H : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = xr[i];
+    if (dr) { v += to_float(dr[i]); xr[i] = v; }
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  T* o1 = out1 + (size_t)blockIdx.x * H;
+  T* o2 = out2 + (size_t)blockIdx.x * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {   // each thread reads back what it wrote itself
+    const float v = xr[i] * inv;
+    o1[i] = from_float<T>(w1[i] * v);
+    o2[i] = from_float<T>(w2[i] * v);
+  }
+}
+
+extern "C" int ms_rms_norm_pair(float* x, const void* delta, int delta_dtype, const float* w1, const float* w2, void* out1,
+                                void* out2, int n_rows, int hidden, float eps, int dtype, hipStream_t stream) {
+  if (n_rows <= 0) return MS_OK;
+  if (hidden <= 0) return MS_BAD_ARG;
+  dim3 grid(n_rows), block(hidden >= 1024 ? 256 : 128);
+#define LAUNCH(T, TD) rms_norm_pair_kernel<T, TD><<<grid, block, 0, stream>>>(x, (const TD*)delta, w1, w2, (T*)out1, (T*)out2, hidden, eps)
+  if (dtype == MS_F32) {
+    if (delta && delta_dtype == MS_BF16) return MS_BAD_ARG;
+    LAUNCH(float, float);
+  } else if (dtype == MS_BF16) {
+    if (delta && delta_dtype == MS_F32) LAUNCH(bf16, float);
+    else LAUNCH(bf16, bf16);
+  } else return MS_BAD_ARG;
+#undef LAUNCH
+  return ms_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
 // x[n, :] += delta[n, :]  (the residual sum alone, for arrangements that do not fuse it into a norm)
 template <typename TD>
 __global__ void residual_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, size_t total) {

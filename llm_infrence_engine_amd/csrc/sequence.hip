@@ -20,10 +20,10 @@ __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf
 // mode 0: the sum; 1: x + the sum; 2: silu of the sum.
 template <typename T>
 __global__ void short_conv_kernel(const T* __restrict__ x, size_t x_stride, const float* __restrict__ w,
-                                  const T* __restrict__ state, const int* __restrict__ token_req,
+                                  const T* state, const int* __restrict__ token_req,
                                   const int* __restrict__ q_start, const int* __restrict__ state_slots,
                                   const int* __restrict__ n_live_tokens, T* __restrict__ out, size_t out_stride,
-                                  int C, int taps, int mode) {
+                                  int C, int taps, int mode, T* state_out) {
   const int n = blockIdx.x;
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= C) return;
@@ -41,6 +41,18 @@ __global__ void short_conv_kernel(const T* __restrict__ x, size_t x_stride, cons
   if (mode == 1) acc += to_float(x[(size_t)n * x_stride + c]);
   else if (mode == 2) acc = acc * sigmoid_f(acc);
   out[(size_t)n * out_stride + c] = from_float<T>(acc);
+  if (state_out) {
+    // a step of single tokens: this thread is the only one that reads or writes its request's state of this channel,
+    // so it moves the state on itself (one place up, the token's input last) and no second kernel is needed
+    T* so = state_out + (size_t)state_slots[r] * (taps - 1) * C;
+    T keep[MAX_TAPS];
+#pragma unroll
+    for (int i = 0; i < MAX_TAPS - 1; ++i)
+      if (i < taps - 1) keep[i] = i + 1 < taps - 1 ? so[(size_t)(i + 1) * C + c] : x[(size_t)n * x_stride + c];
+#pragma unroll
+    for (int i = 0; i < MAX_TAPS - 1; ++i)
+      if (i < taps - 1) so[(size_t)i * C + c] = keep[i];
+  }
 }
 
 // After the convolution: the state of every request with tokens becomes its last taps - 1 inputs.
@@ -130,7 +142,8 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
   // to memory serves a whole chunk and is over by the time the chunk before has been walked.
   constexpr int LT = Dp > 256 ? 64 : 16, EPL = (Dp + LT - 1) / LT, VPL = SINGLE ? 1 : 16 / LPC;   // a chunk has at most 16 / LPC values of v a lane   // a whole wave to a token of the longest keys
   const int tl = tid / LT, l16 = tid % LT;
-  float qf[EPL], kf[EPL], af[EPL], vf[VPL], bf = 0.f;
+  T qr[EPL], kr[EPL], vr[VPL], br = from_float<T>(0.f);   // as loaded: nothing waits for them before the staging
+  float ar[EPL], dr[EPL];
   auto ask = [&](int c0) __attribute__((always_inline)) {
     const int cn = min(chunk, L - c0);
     if (tl < cn) {
@@ -142,18 +155,16 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
       for (int e = 0; e < EPL; ++e) {
         const int i = l16 + e * LT;
         const bool in = i < D;
-        qf[e] = in ? to_float(qp[i]) : 0.f;
-        kf[e] = in ? to_float(kp[i]) : 0.f;
-        af[e] = in ? ap[i] + dt_bias[(size_t)h * D + i] : 0.f;
+        if (in) { qr[e] = qp[i]; kr[e] = kp[i]; ar[e] = ap[i]; dr[e] = dt_bias[(size_t)h * D + i]; }
       }
-      if (l16 == 0) bf = to_float(b[n * b_stride + h]);
+      if (l16 == 0) br = b[n * b_stride + h];
     }
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       const int e = tid + j * blockDim.x;
       if (e < cn * cols_per_block) {
         const int t = e / cols_per_block, jj = e - t * cols_per_block;
-        vf[j] = col0 + jj < E ? to_float(v[(size_t)(s0 + c0 + t) * qkv_stride + (size_t)h * E + col0 + jj]) : 0.f;
+        if (col0 + jj < E) vr[j] = v[(size_t)(s0 + c0 + t) * qkv_stride + (size_t)h * E + col0 + jj];
       }
     }
   };
@@ -164,9 +175,16 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
     if (!ASK_AHEAD) ask(c0);
     __syncthreads();   // the chunk before is done with the staging area
     if (tl < cn) {
-      float sq = 0.f, sk = 0.f;
+      float sq = 0.f, sk = 0.f, qf[EPL], kf[EPL], af[EPL];
 #pragma unroll
-      for (int e = 0; e < EPL; ++e) { sq = fmaf(qf[e], qf[e], sq); sk = fmaf(kf[e], kf[e], sk); }
+      for (int e = 0; e < EPL; ++e) {
+        const bool in = l16 + e * LT < D;
+        qf[e] = in ? to_float(qr[e]) : 0.f;
+        kf[e] = in ? to_float(kr[e]) : 0.f;
+        af[e] = in ? ar[e] + dr[e] : 0.f;
+        sq = fmaf(qf[e], qf[e], sq);
+        sk = fmaf(kf[e], kf[e], sk);
+      }
       sq = LT == 64 ? wave_sum(sq) : group_sum<16>(sq);
       sk = LT == 64 ? wave_sum(sk) : group_sum<16>(sk);
       const float iq = q_scale / sqrtf(sq + 1e-6f), ik = 1.0f / sqrtf(sk + 1e-6f);
@@ -180,12 +198,15 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
           gs[tl * Dp + i] = in ? expf(-rate * softplus_f(af[e])) : 1.f;
         }
       }
-      if (l16 == 0) bs[tl] = sigmoid_f(bf);
+      if (l16 == 0) bs[tl] = sigmoid_f(to_float(br));
     }
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       const int e = tid + j * blockDim.x;
-      if (e < cn * cols_per_block) vs[e] = vf[j];
+      if (e < cn * cols_per_block) {
+        const int t = e / cols_per_block, jj = e - t * cols_per_block;
+        vs[e] = col0 + jj < E ? to_float(vr[j]) : 0.f;
+      }
     }
     __syncthreads();
     if (ASK_AHEAD && c0 + chunk < L) ask(c0 + chunk);
@@ -303,7 +324,7 @@ __global__ void xielu_kernel(const T* __restrict__ x, const float* __restrict__ 
 extern "C" int ms_short_conv(const void* x, long long x_stride, const float* w, void* state, const int* token_req,
                              const int* q_start, const int* state_slots, const int* n_live_tokens, void* out,
                              long long out_stride, int n_tokens, int n_requests, int channels, int taps, int mode,
-                             int update_state, int dtype, hipStream_t stream) {
+                             int update_state, int single_tokens, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
   if (channels <= 0 || taps < 1 || mode < 0 || mode > 2 || n_requests <= 0) return MS_BAD_ARG;
   if (taps > MAX_TAPS) return MS_UNSUPPORTED;
@@ -313,10 +334,11 @@ extern "C" int ms_short_conv(const void* x, long long x_stride, const float* w, 
   dim3 block(threads), grid(n_tokens, cblocks), ugrid(cblocks, n_requests);
 #define LAUNCH(T)                                                                                                       \
   do {                                                                                                                  \
+    const bool fused = update_state && single_tokens && taps > 1;                                                       \
     short_conv_kernel<T><<<grid, block, 0, stream>>>((const T*)x, (size_t)x_stride, w, (const T*)state, token_req,     \
                                                      q_start, state_slots, n_live_tokens, (T*)out, (size_t)out_stride, \
-                                                     channels, taps, mode);                                             \
-    if (update_state && taps > 1)                                                                                       \
+                                                     channels, taps, mode, fused ? (T*)state : nullptr);               \
+    if (update_state && taps > 1 && !fused)                                                                             \
       short_conv_update_kernel<T><<<ugrid, block, 0, stream>>>((const T*)x, (size_t)x_stride, (T*)state, q_start,      \
                                                                state_slots, channels, taps);                            \
   } while (0)

@@ -23,6 +23,7 @@ _SIGNATURES = {
     "ms_embed": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_rms_norm": [_c_ptr, _c_ptr, _c_int, _c_int, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int,
                     _c_int, _c_ptr],
+    "ms_rms_norm_pair": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "ms_gemm_skinny_norm": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int,
                             _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_qkv_rope_store": [_c_ptr, _c_ll, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
@@ -73,7 +74,7 @@ _SIGNATURES = {
                   _c_ptr],
     "ms_sample_workspace_bytes": [_c_int],
     "ms_short_conv": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int,
-                      _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gated_delta": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gated_head_norm": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
@@ -214,6 +215,25 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tenso
     _call("ms_rms_norm", x.data_ptr(), _ptr(delta), dcode, n_partials, N * H, weight.data_ptr(), _ptr(rows),
           out.data_ptr(), n_rows, H, float(eps), int(write_back), _code(out.dtype), _stream())
     return out
+
+
+def rms_norm_pair(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, eps: float, out1: torch.Tensor, out2: torch.Tensor,
+                  delta: Optional[torch.Tensor] = None):
+    """out1 = w1 * normalised(x (+ delta)), out2 = w2 * normalised(x (+ delta)): two norms of the same rows of the float
+    residual stream in one pass; with ``delta`` [N, H] the sum is written back to x."""
+    _check(x, "x", torch.float32)
+    N, H = x.shape
+    _check(w1, "w1", torch.float32, (H,))
+    _check(w2, "w2", torch.float32, (H,))
+    _check(out1, "out1", None, (N, H))
+    _check(out2, "out2", out1.dtype, (N, H))
+    dcode = 0
+    if delta is not None:
+        _check(delta, "delta", None, (N, H))
+        dcode = _code(delta.dtype)
+    _call("ms_rms_norm_pair", x.data_ptr(), _ptr(delta), dcode, w1.data_ptr(), w2.data_ptr(), out1.data_ptr(),
+          out2.data_ptr(), N, H, float(eps), _code(out1.dtype), _stream())
+    return out1, out2
 
 
 def bias_add(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
@@ -877,7 +897,7 @@ def short_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx, 
     _check(ctx.state_slots, "state_slots", torch.int32, (R,))
     _call("ms_short_conv", x.data_ptr(), xs, weight.data_ptr(), state.data_ptr(), ctx.token_req.data_ptr(),
           ctx.q_start.data_ptr(), ctx.state_slots.data_ptr(), _ptr(ctx.n_live_tokens), out.data_ptr(), os_, N, R, C, taps,
-          mode, int(update_state), _code(x.dtype), _stream())
+          mode, int(update_state), int(getattr(ctx, "max_q_len", 0) == 1), _code(x.dtype), _stream())
     return out
 
 

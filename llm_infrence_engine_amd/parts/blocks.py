@@ -32,8 +32,12 @@ class ParallelResidual(Block):
     optional = ("position", "input_filter", "feed_forward_norm", "feed_forward")
 
     def forward(self, x, pending, ctx, kv, state):
-        h = self.mixer_norm.forward(x, delta=pending)          # x now holds the sum both branches read
-        h2 = self.feed_forward_norm.forward(x) if self.feed_forward is not None else None
+        # x holds the sum both branches read before either adds to it; the two norms share their pass over x
+        if self.feed_forward is not None and hasattr(self.mixer_norm, "forward_pair"):
+            h, h2 = self.mixer_norm.forward_pair(self.feed_forward_norm, x, delta=pending)
+        else:
+            h = self.mixer_norm.forward(x, delta=pending)
+            h2 = self.feed_forward_norm.forward(x) if self.feed_forward is not None else None
         if self.input_filter is not None:
             h = self.input_filter.forward(h, ctx, self.state_of("input_filter", state))
         a = self.mixer.forward_residual(h, ctx, kv, self.state_of("mixer", state), x)

@@ -34,6 +34,17 @@ class RMSNorm(Norm):
         return ops.rms_norm(x, self.weight, self.eps, out, delta=delta, rows=rows, write_back=write_back)
 
 
+    def forward_pair(self, other: "RMSNorm", x, delta=None):
+        """(self's norm, ``other``'s norm) of the same rows of x (+ delta, kept in x): one pass when the two differ in
+        their scales only, else two."""
+        if not isinstance(other, RMSNorm) or other.size != self.size or other.eps != self.eps or \
+                (delta is not None and delta.dim() != 2):
+            first = self.forward(x, delta)
+            return first, other.forward(x)
+        n = x.shape[0]
+        return ops.rms_norm_pair(x, self.weight, other.weight, self.eps, self.rt.empty(n, self.size),
+                                 self.rt.empty(n, self.size), delta=delta)
+
     def lazy(self, x, delta=None, rows=None, write_back=True):
         """As ``forward``, for a consumer that can fold the norm into its first product: with few rows in
         bfloat16 the addend is summed into x now and the normalisation is left to that product."""
