@@ -119,11 +119,38 @@ extern "C" int ms_rms_norm(float* x, const void* delta, int delta_dtype, int n_p
 template <typename T, typename TD>
 __global__ void rms_norm_pair_kernel(float* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ w1,
                                      const float* __restrict__ w2, T* __restrict__ out1, T* __restrict__ out2, int H,
-                                     float eps) {
+                                     float eps, int staged) {
   __shared__ float red[16];
+  extern __shared__ float buf[];   // H floats when staged: the row after the residual sum
   float* xr = x + (size_t)blockIdx.x * H;
   const TD* dr = delta ? delta + (size_t)blockIdx.x * H : nullptr;
+  T* o1 = out1 + (size_t)blockIdx.x * H;
+  T* o2 = out2 + (size_t)blockIdx.x * H;
   float ss = 0.f;
+  if (staged && H % 4 == 0) {      // four values at a time (rows start 16-byte aligned when H % 4 == 0)
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      float4 v = *reinterpret_cast<const float4*>(xr + i);
+      if (dr) {
+        v.x += to_float(dr[i]); v.y += to_float(dr[i + 1]); v.z += to_float(dr[i + 2]); v.w += to_float(dr[i + 3]);
+        *reinterpret_cast<float4*>(xr + i) = v;
+      }
+      *reinterpret_cast<float4*>(buf + i) = v;
+      ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      const float4 v = *reinterpret_cast<const float4*>(buf + i);
+      const float4 a = *reinterpret_cast<const float4*>(w1 + i);
+      const float4 b = *reinterpret_cast<const float4*>(w2 + i);
+      const float n0 = v.x * inv, n1 = v.y * inv, n2 = v.z * inv, n3 = v.w * inv;
+      o1[i] = from_float<T>(a.x * n0); o1[i + 1] = from_float<T>(a.y * n1);
+      o1[i + 2] = from_float<T>(a.z * n2); o1[i + 3] = from_float<T>(a.w * n3);
+      o2[i] = from_float<T>(b.x * n0); o2[i + 1] = from_float<T>(b.y * n1);
+      o2[i + 2] = from_float<T>(b.z * n2); o2[i + 3] = from_float<T>(b.w * n3);
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float v = xr[i];
     if (dr) { v += to_float(dr[i]); xr[i] = v; }
@@ -131,8 +158,6 @@ __global__ void rms_norm_pair_kernel(float* __restrict__ x, const TD* __restrict
   }
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)H + eps);
-  T* o1 = out1 + (size_t)blockIdx.x * H;
-  T* o2 = out2 + (size_t)blockIdx.x * H;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {   // each thread reads back what it wrote itself
     const float v = xr[i] * inv;
     o1[i] = from_float<T>(w1[i] * v);
@@ -145,7 +170,9 @@ extern "C" int ms_rms_norm_pair(float* x, const void* delta, int delta_dtype, co
   if (n_rows <= 0) return MS_OK;
   if (hidden <= 0) return MS_BAD_ARG;
   dim3 grid(n_rows), block(hidden >= 1024 ? 256 : 128);
-#define LAUNCH(T, TD) rms_norm_pair_kernel<T, TD><<<grid, block, 0, stream>>>(x, (const TD*)delta, w1, w2, (T*)out1, (T*)out2, hidden, eps)
+  const int staged = (size_t)hidden * sizeof(float) + 64 <= 65536 ? 1 : 0;
+  const size_t lds = staged ? (size_t)hidden * sizeof(float) : 0;
+#define LAUNCH(T, TD) rms_norm_pair_kernel<T, TD><<<grid, block, lds, stream>>>(x, (const TD*)delta, w1, w2, (T*)out1, (T*)out2, hidden, eps, staged)
   if (dtype == MS_F32) {
     if (delta && delta_dtype == MS_BF16) return MS_BAD_ARG;
     LAUNCH(float, float);

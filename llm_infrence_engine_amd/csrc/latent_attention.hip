@@ -18,7 +18,8 @@ __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf
 // ------------------------------------------------------------------------------------------------
 // out[n, h, j] = sum_i in[n, h, i] * M[h, i, j] (* sigmoid(gate[n, h, j])).  A block owns TM tokens of one head and 64
 // consecutive j; its four waves each take a quarter of the i (rows of M, read coalesced, eight in flight) and their
-// sums are added through LDS in wave order.  TM is 8 for few tokens (more blocks) and 16 for many (M is read half as often).
+// sums are added through LDS in wave order: the shape for few tokens (a decode step), where blocks are few and a
+// thread's walk over all the i would be the longest chain of the step.
 constexpr int HM_WAVES = 4;
 
 template <typename T, typename TO, int TM>
@@ -65,6 +66,44 @@ head_matmul_kernel(const T* __restrict__ in, size_t in_tok, size_t in_head, cons
     if (n0 + t >= N) break;
     float y = acc[t];
     for (int w = 0; w < HM_WAVES - 1; ++w) y += part[(w * TM + t) * MS_WAVE + lane];
+    if (gate) y *= sigmoid_f(to_float(gate[(size_t)(n0 + t) * gate_tok + (size_t)h * J + j]));
+    out[(size_t)(n0 + t) * out_tok + (size_t)h * out_head + j] = from_float<TO>(y);
+  }
+}
+
+// The same product for many tokens: a block owns 8 tokens of one head and up to 256 consecutive j, a thread all the i
+// of its j; the blocks are many, and each reads its tokens once.
+constexpr int HM_TOKENS = 8;
+
+template <typename T, typename TO>
+__global__ void head_matmul_wide_kernel(const T* __restrict__ in, size_t in_tok, size_t in_head, const T* __restrict__ M,
+                                        TO* __restrict__ out, size_t out_tok, size_t out_head, const T* __restrict__ gate,
+                                        size_t gate_tok, int N, int I, int J) {
+  extern __shared__ __align__(16) float xs[];   // [I][HM_TOKENS]
+  const int h = blockIdx.y, n0 = blockIdx.x * HM_TOKENS;
+  const int j = blockIdx.z * blockDim.x + threadIdx.x;
+  for (int e = threadIdx.x; e < I * HM_TOKENS; e += blockDim.x) {
+    const int t = e / I, i = e - t * I;
+    xs[i * HM_TOKENS + t] = n0 + t < N ? to_float(in[(size_t)(n0 + t) * in_tok + (size_t)h * in_head + i]) : 0.f;
+  }
+  __syncthreads();
+  if (j >= J) return;
+  float acc[HM_TOKENS];
+#pragma unroll
+  for (int t = 0; t < HM_TOKENS; ++t) acc[t] = 0.f;
+  const T* Mh = M + (size_t)h * I * J + j;
+#pragma unroll 8
+  for (int i = 0; i < I; ++i) {   // eight rows of M in flight: the loop waits for memory, not for arithmetic
+    const float m = to_float(Mh[(size_t)i * J]);
+    const float4 a = *reinterpret_cast<const float4*>(xs + i * HM_TOKENS);
+    const float4 b = *reinterpret_cast<const float4*>(xs + i * HM_TOKENS + 4);
+    acc[0] = fmaf(a.x, m, acc[0]); acc[1] = fmaf(a.y, m, acc[1]); acc[2] = fmaf(a.z, m, acc[2]); acc[3] = fmaf(a.w, m, acc[3]);
+    acc[4] = fmaf(b.x, m, acc[4]); acc[5] = fmaf(b.y, m, acc[5]); acc[6] = fmaf(b.z, m, acc[6]); acc[7] = fmaf(b.w, m, acc[7]);
+  }
+#pragma unroll
+  for (int t = 0; t < HM_TOKENS; ++t) {
+    if (n0 + t >= N) break;
+    float y = acc[t];
     if (gate) y *= sigmoid_f(to_float(gate[(size_t)(n0 + t) * gate_tok + (size_t)h * J + j]));
     out[(size_t)(n0 + t) * out_tok + (size_t)h * out_head + j] = from_float<TO>(y);
   }
@@ -242,19 +281,30 @@ extern "C" int ms_head_matmul(const void* in, long long in_tok, long long in_hea
                               int heads, int I, int J, int dtype, int out_dtype, hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
   if (heads <= 0 || I <= 0 || J <= 0) return MS_BAD_ARG;
-  int tm = n_tokens >= 256 ? 16 : 8;
-  if (tm == 16 && ((size_t)I * 16 + (size_t)(HM_WAVES - 1) * 16 * MS_WAVE) * sizeof(float) > 65536) tm = 8;
+  // float: always the one order of summation, whatever the step holds
+  if (n_tokens > 64 || dtype == MS_F32) {
+    const size_t lds = (size_t)I * HM_TOKENS * sizeof(float);
+    if (lds > 65536 || heads > 65535) return MS_UNSUPPORTED;
+    const int threads = J >= 256 ? 256 : ((J + MS_WAVE - 1) / MS_WAVE) * MS_WAVE;
+    dim3 grid((n_tokens + HM_TOKENS - 1) / HM_TOKENS, heads, (J + threads - 1) / threads), block(threads);
+#define LAUNCH(T, TO) head_matmul_wide_kernel<T, TO><<<grid, block, lds, stream>>>((const T*)in, (size_t)in_tok, (size_t)in_head, (const T*)M, (TO*)out, (size_t)out_tok, (size_t)out_head, (const T*)gate, (size_t)gate_tok, n_tokens, I, J)
+    if (dtype == MS_F32 && out_dtype == MS_F32) LAUNCH(float, float);
+    else if (dtype == MS_BF16 && out_dtype == MS_BF16) LAUNCH(bf16, bf16);
+    else if (dtype == MS_BF16 && out_dtype == MS_F32) LAUNCH(bf16, float);
+    else return MS_BAD_ARG;
+#undef LAUNCH
+    return ms_launch_status();
+  }
+  constexpr int tm = 8;
   const size_t lds = ((size_t)I * tm + (size_t)(HM_WAVES - 1) * tm * MS_WAVE) * sizeof(float);
   if (lds > 65536 || heads > 65535 || (J + MS_WAVE - 1) / MS_WAVE > 65535) return MS_UNSUPPORTED;
   dim3 grid((n_tokens + tm - 1) / tm, heads, (J + MS_WAVE - 1) / MS_WAVE), block(HM_WAVES * MS_WAVE);
-#define LAUNCH1(T, TO, TM) head_matmul_kernel<T, TO, TM><<<grid, block, lds, stream>>>((const T*)in, (size_t)in_tok, (size_t)in_head, (const T*)M, (TO*)out, (size_t)out_tok, (size_t)out_head, (const T*)gate, (size_t)gate_tok, n_tokens, I, J)
-#define LAUNCH(T, TO) do { if (tm == 16) LAUNCH1(T, TO, 16); else LAUNCH1(T, TO, 8); } while (0)
+#define LAUNCH(T, TO) head_matmul_kernel<T, TO, 8><<<grid, block, lds, stream>>>((const T*)in, (size_t)in_tok, (size_t)in_head, (const T*)M, (TO*)out, (size_t)out_tok, (size_t)out_head, (const T*)gate, (size_t)gate_tok, n_tokens, I, J)
   if (dtype == MS_F32 && out_dtype == MS_F32) LAUNCH(float, float);
   else if (dtype == MS_BF16 && out_dtype == MS_BF16) LAUNCH(bf16, bf16);
   else if (dtype == MS_BF16 && out_dtype == MS_F32) LAUNCH(bf16, float);
   else return MS_BAD_ARG;
 #undef LAUNCH
-#undef LAUNCH1
   return ms_launch_status();
 }
 
