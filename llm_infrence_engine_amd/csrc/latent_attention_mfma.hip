@@ -85,19 +85,21 @@ latent_attention_mfma_kernel(const bf16* __restrict__ q, size_t q_tok, size_t q_
       const int page = kb <= key_hi ? __builtin_amdgcn_readfirstlane(table[kb / page_size]) : 0;
       row0[u] = (size_t)page * page_size + (kb <= key_hi ? kb % page_size : 0);
     }
-    // scores: s[u] holds keys base + u*16 + kq*4 + (0..3) of this lane's column
+    // scores: s[u] holds keys base + u*16 + kq*4 + (0..3) of this lane's column.  All of a half's key fragments are
+    // asked for before the first product, so that a half costs one trip to memory and not one per fragment.
     f32x4 s[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      bf16x8 kf[KS_C + KS_R];
       const bf16* kp = c_pages + (row0[u] + col16) * C + kq * 8;
-#pragma unroll
-      for (int ks = 0; ks < KS_C; ++ks)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(kp + ks * 32), qv[ks], acc, 0, 0, 0);
       const bf16* rp = r_pages + (row0[u] + col16) * R + kq * 8;
 #pragma unroll
-      for (int ks = 0; ks < KS_R; ++ks)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(rp + ks * 32), qv[KS_C + ks], acc, 0, 0, 0);
+      for (int ks = 0; ks < KS_C; ++ks) kf[ks] = *reinterpret_cast<const bf16x8*>(kp + ks * 32);
+#pragma unroll
+      for (int ks = 0; ks < KS_R; ++ks) kf[KS_C + ks] = *reinterpret_cast<const bf16x8*>(rp + ks * 32);
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS_C + KS_R; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qv[ks], acc, 0, 0, 0);
       s[u] = acc;
     }
     // mask, block maximum
@@ -133,22 +135,30 @@ latent_attention_mfma_kernel(const bf16* __restrict__ q, size_t q_tok, size_t q_
     const bool tail = base + 31 > key_hi;
     const bf16* vp0 = ct_pages + (row0[0] / page_size) * (size_t)page_size * C + row0[0] % page_size + kq * 4;
     const bf16* vp1 = ct_pages + (row0[1] / page_size) * (size_t)page_size * C + row0[1] % page_size + kq * 4;
+    constexpr int VG = 8;      // tiles of 16 entries whose values are asked for together
 #pragma unroll
-    for (int t = 0; t < CT; ++t) {
-      const size_t at = (size_t)(t * 16 + col16) * page_size;
-      const bf16x4 a = *reinterpret_cast<const bf16x4*>(vp0 + at);
-      const bf16x4 b = *reinterpret_cast<const bf16x4*>(vp1 + at);
-      bf16x8 vv;
+    for (int t0 = 0; t0 < CT; t0 += VG) {
+      bf16x4 va[VG], vb[VG];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { vv[i] = a[i]; vv[4 + i] = b[i]; }
-      if (tail) {      // what a reused page still holds past the last visible key must not meet the zero weights
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if (base + kq * 4 + i > key_hi) vv[i] = (__bf16)0.0f;
-          if (base + 16 + kq * 4 + i > key_hi) vv[4 + i] = (__bf16)0.0f;
-        }
+      for (int j = 0; j < VG; ++j) {
+        const size_t at = (size_t)((t0 + j) * 16 + col16) * page_size;
+        va[j] = *reinterpret_cast<const bf16x4*>(vp0 + at);
+        vb[j] = *reinterpret_cast<const bf16x4*>(vp1 + at);
       }
-      o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, p, o[t], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < VG; ++j) {
+        bf16x8 vv;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { vv[i] = va[j][i]; vv[4 + i] = vb[j][i]; }
+        if (tail) {      // what a reused page still holds past the last visible key must not meet the zero weights
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (base + kq * 4 + i > key_hi) vv[i] = (__bf16)0.0f;
+            if (base + 16 + kq * 4 + i > key_hi) vv[4 + i] = (__bf16)0.0f;
+          }
+        }
+        o[t0 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, p, o[t0 + j], 0, 0, 0);
+      }
     }
   }
   float l = lsum[0];      // every row of the product with ones is the column's sum
