@@ -85,22 +85,27 @@ latent_attention_mfma_kernel(const bf16* __restrict__ q, size_t q_tok, size_t q_
       const int page = kb <= key_hi ? __builtin_amdgcn_readfirstlane(table[kb / page_size]) : 0;
       row0[u] = (size_t)page * page_size + (kb <= key_hi ? kb % page_size : 0);
     }
-    // scores: s[u] holds keys base + u*16 + kq*4 + (0..3) of this lane's column.  All of a half's key fragments are
-    // asked for before the first product, so that a half costs one trip to memory and not one per fragment.
+    // scores: s[u] holds keys base + u*16 + kq*4 + (0..3) of this lane's column.  All key fragments of the block are
+    // asked for before the first product, so that a block costs one trip to memory for its keys, not one per fragment.
     f32x4 s[2];
+    {
+      bf16x8 kf[2][KS_C + KS_R];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      bf16x8 kf[KS_C + KS_R];
-      const bf16* kp = c_pages + (row0[u] + col16) * C + kq * 8;
-      const bf16* rp = r_pages + (row0[u] + col16) * R + kq * 8;
+      for (int u = 0; u < 2; ++u) {
+        const bf16* kp = c_pages + (row0[u] + col16) * C + kq * 8;
+        const bf16* rp = r_pages + (row0[u] + col16) * R + kq * 8;
 #pragma unroll
-      for (int ks = 0; ks < KS_C; ++ks) kf[ks] = *reinterpret_cast<const bf16x8*>(kp + ks * 32);
+        for (int ks = 0; ks < KS_C; ++ks) kf[u][ks] = *reinterpret_cast<const bf16x8*>(kp + ks * 32);
 #pragma unroll
-      for (int ks = 0; ks < KS_R; ++ks) kf[KS_C + ks] = *reinterpret_cast<const bf16x8*>(rp + ks * 32);
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int ks = 0; ks < KS_R; ++ks) kf[u][KS_C + ks] = *reinterpret_cast<const bf16x8*>(rp + ks * 32);
+      }
 #pragma unroll
-      for (int ks = 0; ks < KS_C + KS_R; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qv[ks], acc, 0, 0, 0);
-      s[u] = acc;
+      for (int u = 0; u < 2; ++u) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS_C + KS_R; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qv[ks], acc, 0, 0, 0);
+        s[u] = acc;
+      }
     }
     // mask, block maximum
     float bm = -INFINITY;
@@ -135,7 +140,7 @@ latent_attention_mfma_kernel(const bf16* __restrict__ q, size_t q_tok, size_t q_
     const bool tail = base + 31 > key_hi;
     const bf16* vp0 = ct_pages + (row0[0] / page_size) * (size_t)page_size * C + row0[0] % page_size + kq * 4;
     const bf16* vp1 = ct_pages + (row0[1] / page_size) * (size_t)page_size * C + row0[1] % page_size + kq * 4;
-    constexpr int VG = 8;      // tiles of 16 entries whose values are asked for together
+    constexpr int VG = CT < 16 ? CT : 16;      // tiles of 16 entries whose values are asked for together
 #pragma unroll
     for (int t0 = 0; t0 < CT; t0 += VG) {
       bf16x4 va[VG], vb[VG];
