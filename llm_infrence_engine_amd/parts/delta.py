@@ -22,7 +22,9 @@ from .base import Mixer, StateNeed, register_part
 def _rows(t: torch.Tensor, lo: int, hi: int) -> torch.Tensor:
     """Columns lo..hi of ``t`` as the input of a product: the slice itself where a kernel takes it as it lies."""
     s = t[:, lo:hi]
-    if t.dtype == torch.float32 or (t.shape[0] <= ops.SKINNY_MAX_ROWS and ops.skinny_ok(s, s)):
+    # the float kernel takes any row slice; the few-rows matrix-core kernels take rows that start 16-byte aligned
+    if t.dtype == torch.float32 or (t.shape[0] <= ops.SKINNY_MAX_ROWS and s.shape[1] % 8 == 0
+                                    and (t.shape[0] == 1 or s.stride(0) % 8 == 0) and s.data_ptr() % 16 == 0):
         return s
     return s.contiguous()
 
