@@ -105,8 +105,11 @@ constexpr int DELTA_CHUNK = 16;
 
 // SINGLE: every request of the step has one token (a decode step).  Nothing is asked or fetched ahead then, which
 // leaves registers for three blocks to a CU: the step is the read and the write of the states, and needs them in flight.
-template <typename T, int DPT, int LPC, bool SINGLE>
-__global__ void __launch_bounds__(256, SINGLE ? 3 : 1)
+// SPLIT: the block has twice the threads; the first half walks the tokens of a chunk while the second half stages
+// the next chunk into a second set of buffers (its arithmetic, the unit norms and the decays' exponentials, is as long
+// as the walk over a chunk and shares nothing with it), so a chunk costs the longer of the two and one barrier.
+template <typename T, int DPT, int LPC, bool SINGLE, bool SPLIT>
+__global__ void __launch_bounds__(SPLIT ? 512 : 256, SINGLE ? 3 : 1)
 gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, size_t qkv_stride,
                    const float* __restrict__ a, const T* __restrict__ b, size_t b_stride,
                    const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ state,
@@ -115,18 +118,25 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
   extern __shared__ __align__(16) float lds[];
   constexpr int lpc = LPC;
   constexpr int Dp = DPT * LPC;             // padded key size
-  float* qs = lds;                          // [chunk][Dp]
-  float* ks = qs + chunk * Dp;
-  float* gs = ks + chunk * Dp;
-  float* vs = gs + chunk * Dp;              // [chunk][cols_per_block]
-  float* bs = vs + chunk * cols_per_block;  // [chunk]
+  float *qs, *ks, *gs, *vs, *bs;            // [chunk][Dp] three times, [chunk][cols_per_block], [chunk]
+  const int buf_floats = (chunk * (3 * Dp + cols_per_block + 1) + 3) / 4 * 4;
+  auto use_buffers = [&](int which) __attribute__((always_inline)) {
+    qs = lds + (size_t)which * buf_floats;
+    ks = qs + chunk * Dp;
+    gs = ks + chunk * Dp;
+    vs = gs + chunk * Dp;
+    bs = vs + chunk * cols_per_block;
+  };
+  use_buffers(0);
   const int r = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * cols_per_block;
   const int kvh = h / (H / G);
   const int s0 = q_start[r], L = q_start[r + 1] - s0;
   if (L <= 0) return;
-  const int tid = threadIdx.x, lane = tid & (MS_WAVE - 1), wave = tid / MS_WAVE, nwaves = blockDim.x / MS_WAVE;
+  const int nth = SPLIT ? blockDim.x / 2 : blockDim.x;      // threads of a role
+  const bool producer = SPLIT && (int)threadIdx.x >= nth;
+  const int tid = producer ? threadIdx.x - nth : threadIdx.x;   // the thread's place within its role
   const int part = tid % lpc, col = col0 + tid / lpc;
-  const bool live = col < E && tid / lpc < cols_per_block;
+  const bool live = !producer && col < E && tid / lpc < cols_per_block;
   float* Sg = state + (((size_t)state_slots[r] * H + h) * D) * E;
   float S[DPT];
 #pragma unroll
@@ -161,7 +171,7 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
     }
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
-      const int e = tid + j * blockDim.x;
+      const int e = tid + j * nth;
       if (e < cn * cols_per_block) {
         const int t = e / cols_per_block, jj = e - t * cols_per_block;
         if (col0 + jj < E) vr[j] = v[(size_t)(s0 + c0 + t) * qkv_stride + (size_t)h * E + col0 + jj];
@@ -169,11 +179,8 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
     }
   };
   constexpr bool ASK_AHEAD = DPT <= 32 && !SINGLE;   // the longest columns leave no registers to hold a chunk through the walk
-  if (ASK_AHEAD) ask(0);
-  for (int c0 = 0; c0 < L; c0 += chunk) {
+  auto stage = [&](int c0) __attribute__((always_inline)) {
     const int cn = min(chunk, L - c0);
-    if (!ASK_AHEAD) ask(c0);
-    __syncthreads();   // the chunk before is done with the staging area
     if (tl < cn) {
       float sq = 0.f, sk = 0.f, qf[EPL], kf[EPL], af[EPL];
 #pragma unroll
@@ -202,14 +209,15 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
     }
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
-      const int e = tid + j * blockDim.x;
+      const int e = tid + j * nth;
       if (e < cn * cols_per_block) {
         const int t = e / cols_per_block, jj = e - t * cols_per_block;
         vs[e] = col0 + jj < E ? to_float(vr[j]) : 0.f;
       }
     }
-    __syncthreads();
-    if (ASK_AHEAD && c0 + chunk < L) ask(c0 + chunk);
+  };
+  auto walk = [&](int c0) __attribute__((always_inline)) {
+    const int cn = min(chunk, L - c0);
     // the rows of the next token's q, k and g are fetched from LDS while the current token is worked on (two sets of
     // registers taken in turn, so that nothing is copied); the two sums over a column run as four chains each
     struct Rows { float g[DPT], k[DPT], q[DPT]; };
@@ -273,6 +281,38 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
         fetch(ra, t);
         token(ra, t, bs[t], vs[t * cols_per_block + my_col]);
       }
+    }
+  };
+  if (SPLIT) {
+    if (producer) {
+      ask(0);
+      stage(0);
+      if (chunk < L) ask(chunk);
+    }
+    __syncthreads();
+    int which = 0;
+    for (int c0 = 0; c0 < L; c0 += chunk, which ^= 1) {
+      if (producer) {
+        if (c0 + chunk < L) {      // the walkers read the other set; the set written here was last read a barrier ago
+          use_buffers(which ^ 1);
+          stage(c0 + chunk);
+          if (c0 + 2 * chunk < L) ask(c0 + 2 * chunk);
+        }
+      } else {
+        use_buffers(which);
+        walk(c0);
+      }
+      __syncthreads();
+    }
+  } else {
+    if (ASK_AHEAD) ask(0);
+    for (int c0 = 0; c0 < L; c0 += chunk) {
+      if (!ASK_AHEAD) ask(c0);
+      __syncthreads();   // the chunk before is done with the staging area
+      stage(c0);
+      __syncthreads();
+      if (ASK_AHEAD && c0 + chunk < L) ask(c0 + chunk);
+      walk(c0);
     }
   }
 #pragma unroll
@@ -385,16 +425,17 @@ extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long 
   int chunk = DELTA_CHUNK < threads / stagers ? DELTA_CHUNK : threads / stagers;
   const size_t per_token = (3 * (size_t)dpt * lpc + cols + 1) * sizeof(float);
   while (chunk > 1 && chunk * per_token > 65536) chunk /= 2;
-  const size_t lds = chunk * per_token;
+  const size_t lds = ((chunk * per_token / sizeof(float) + 3) / 4 * 4) * sizeof(float);   // one set of buffers
   if (lds > 65536) return MS_UNSUPPORTED;
-#define LAUNCH1(T, DPT, LPC, ONE)                                                                                       \
-  gated_delta_kernel<T, DPT, LPC, ONE><<<grid, block, lds, stream>>>(                                                   \
+#define LAUNCH1(T, DPT, LPC, ONE, TWO)                                                                                  \
+  gated_delta_kernel<T, DPT, LPC, ONE, TWO><<<grid, dim3(threads * ((TWO) ? 2 : 1)), lds * ((TWO) ? 2 : 1), stream>>>(  \
       (const T*)q, (const T*)k, (const T*)v, (size_t)qkv_stride, a, (const T*)b, (size_t)b_stride, A_log, dt_bias,     \
       state, q_start, state_slots, out, heads, kv_heads, dim, vdim, cols, chunk)
 #define LAUNCH(T, DPT, LPC)                                                                                             \
   do {                                                                                                                  \
-    if (single_tokens && DPT <= 16) LAUNCH1(T, DPT, LPC, (DPT <= 16));                                                       \
-    else LAUNCH1(T, DPT, LPC, false);                                                                                   \
+    if (single_tokens && DPT <= 16) LAUNCH1(T, DPT, LPC, (DPT <= 16), false);                                           \
+    else if (DPT <= 16 && 2 * lds <= 65536) LAUNCH1(T, DPT, LPC, false, (DPT <= 16));                                   \
+    else LAUNCH1(T, DPT, LPC, false, false);                                                                            \
   } while (0)
 #define BY_DPT(T)                                                                                                       \
   do {                                                                                                                  \
