@@ -602,6 +602,31 @@ def test_portions_and_batches_change_nothing_in_32_bit(shape, tmp_path):
 
 
 @gpu
+def test_one_row_and_few_pages_serve_every_request_in_turn(shape):
+    """An engine with a single request row and pages for one request: every request gets the state slot and the pages
+    its predecessor left, in portions, and must start from zero state and see none of the old keys."""
+    from llm_infrence_engine_amd.engine.batch import StepEntry
+    from llm_infrence_engine_amd.engine.runner import load_runner
+
+    name, cfg, folder, reqs, want, noise = shape
+    page = PAGES[name]
+    longest = max(len(t) for t in reqs.values())
+    runner = load_runner(folder, dtype="float32", page_size=page, num_pages=-(-longest // page) + 1, max_requests=1,
+                         max_len=-(-longest // page) * page)
+    for rid, toks in reqs.items():
+        cut = max(1, len(toks) // 2)
+        first = runner.step([StepEntry(rid, toks[:cut], list(range(cut)))])
+        assert runner.manager.row(rid) == 0
+        got = [first.cpu().numpy()]
+        if cut < len(toks):
+            got.append(runner.step([StepEntry(rid, toks[cut:], list(range(len(toks) - cut)))]).cpu().numpy())
+        runner.free_request(rid)
+        assert np.abs(np.concatenate(got) - want[rid]).max() < F32_ATOL, rid
+    runner.manager.check_invariants()
+    assert all(g.allocator.pages_granted_again() > 0 for g in runner.manager.groups)
+
+
+@gpu
 def test_far_token_reaches_the_end_through_the_state(tmp_path):
     """A token 400 places back, far outside every window, still moves the last logits (the delta rule's state
     carries it), in the plain model and equally in the engine, whole and decoded token by token."""
