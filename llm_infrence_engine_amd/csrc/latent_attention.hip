@@ -44,8 +44,8 @@ head_matmul_kernel(const T* __restrict__ in, size_t in_tok, size_t in_head, cons
   const int i0 = wave * per, i1 = min(I, i0 + per);
   if (j < J) {
     const T* Mh = M + (size_t)h * I * J + j;
-#pragma unroll 8
-    for (int i = i0; i < i1; ++i) {
+#pragma unroll 32
+    for (int i = i0; i < i1; ++i) {   // thirty-two rows of M in flight: with few blocks a wave's trips to memory are the time
       const float m = to_float(Mh[(size_t)i * J]);
 #pragma unroll
       for (int t = 0; t < TM; t += 4) {
