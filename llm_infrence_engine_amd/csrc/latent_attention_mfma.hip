@@ -274,26 +274,56 @@ latent_attention_mfma_shared_kernel(const bf16* __restrict__ q, size_t q_tok, si
   for (int t = 0; t < CT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   constexpr int KSEG = (C + R) / 8;     // pieces of 16 bytes in a key's row
-  for (int base = (blk_lo / 32) * 32; base <= blk_hi; base += 32) {
-    size_t row0[2];
+  constexpr int THREADS = LM_WAVES * MS_WAVE;
+  constexpr int KPT = (32 * KSEG + THREADS - 1) / THREADS, VPT = C * 4 / THREADS;   // pieces a thread carries
+  // A key block is asked for one block ahead, into registers, and its page ids one block before that: while a block is
+  // multiplied the next one is on its way, and no load waits for a look-up.
+  bf16x8 kreg[KPT], vreg[VPT];
+  int pages[2];
+  auto lookup = [&](int base) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int kb = base + u * 16;
-      const int page = kb <= blk_hi ? __builtin_amdgcn_readfirstlane(table[kb / page_size]) : 0;
-      row0[u] = (size_t)page * page_size + (kb <= blk_hi ? kb % page_size : 0);
+      pages[u] = kb <= blk_hi ? __builtin_amdgcn_readfirstlane(table[kb / page_size]) : 0;
     }
-    __syncthreads();     // everyone is done with the block before
-    for (int seg = threadIdx.x; seg < 32 * KSEG; seg += LM_WAVES * MS_WAVE) {
-      const int key = seg / KSEG, piece = seg - key * KSEG;
-      const size_t row = row0[key >> 4] + (key & 15);
-      const bf16* src = piece < C / 8 ? c_pages + row * C + piece * 8 : r_pages + row * R + (piece - C / 8) * 8;
-      *reinterpret_cast<bf16x8*>(Ks + key * KROW + piece * 8) = *reinterpret_cast<const bf16x8*>(src);
+  };
+  auto issue = [&](int base) __attribute__((always_inline)) {
+    size_t row0[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) row0[u] = (size_t)pages[u] * page_size + (base + u * 16 <= blk_hi ? (base + u * 16) % page_size : 0);
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+      const int seg = threadIdx.x + j * THREADS;
+      if (seg < 32 * KSEG) {
+        const int key = seg / KSEG, piece = seg - key * KSEG;
+        const size_t row = row0[key >> 4] + (key & 15);
+        const bf16* src = piece < C / 8 ? c_pages + row * C + piece * 8 : r_pages + row * R + (piece - C / 8) * 8;
+        kreg[j] = *reinterpret_cast<const bf16x8*>(src);
+      }
     }
-    for (int seg = threadIdx.x; seg < C * 4; seg += LM_WAVES * MS_WAVE) {
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+      const int seg = threadIdx.x + j * THREADS;
       const int u = seg / (C * 2), rem = seg - u * (C * 2), dim = rem >> 1, piece = rem & 1;
       const bf16* src = ct_pages + (row0[u] / page_size) * (size_t)page_size * C + (size_t)dim * page_size +
                         row0[u] % page_size + piece * 8;
-      bf16x8 v = *reinterpret_cast<const bf16x8*>(src);
+      vreg[j] = *reinterpret_cast<const bf16x8*>(src);
+    }
+  };
+  auto commit = [&](int base) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+      const int seg = threadIdx.x + j * THREADS;
+      if (seg < 32 * KSEG) {
+        const int key = seg / KSEG, piece = seg - key * KSEG;
+        *reinterpret_cast<bf16x8*>(Ks + key * KROW + piece * 8) = kreg[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+      const int seg = threadIdx.x + j * THREADS;
+      const int u = seg / (C * 2), rem = seg - u * (C * 2), dim = rem >> 1, piece = rem & 1;
+      bf16x8 v = vreg[j];
       // what a reused page still holds past the block's last key must not meet the zero weights
       const int k0 = base + u * 16 + piece * 8;
       if (k0 + 7 > blk_hi) {
@@ -303,7 +333,81 @@ latent_attention_mfma_shared_kernel(const bf16* __restrict__ q, size_t q_tok, si
       }
       *reinterpret_cast<bf16x8*>(Vs + dim * LS_VROW + u * 16 + piece * 8) = v;
     }
+  };
+  constexpr bool AHEAD = C <= 256;      // at 512 the accumulators and the query leave no registers to carry a block
+  const int first = (blk_lo / 32) * 32;
+  lookup(first);
+  if (AHEAD) {
+    issue(first);
+    if (first + 32 <= blk_hi) lookup(first + 32);
+  }
+  for (int base = first; base <= blk_hi; base += 32) {
+    __syncthreads();     // everyone is done with the block before
+    if (AHEAD) {
+      commit(base);
+    } else {
+      // four pieces in flight at a time, straight into LDS
+      size_t row0[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) row0[u] = (size_t)pages[u] * page_size + (base + u * 16 <= blk_hi ? (base + u * 16) % page_size : 0);
+      if (base + 32 <= blk_hi) lookup(base + 32);     // the next block's page ids travel with this block's keys
+      constexpr int G = 4;
+#pragma unroll
+      for (int j0 = 0; j0 < KPT; j0 += G) {
+        bf16x8 t[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const int seg = threadIdx.x + (j0 + g) * THREADS;
+          if (j0 + g < KPT && seg < 32 * KSEG) {
+            const int key = seg / KSEG, piece = seg - key * KSEG;
+            const size_t row = row0[key >> 4] + (key & 15);
+            t[g] = *reinterpret_cast<const bf16x8*>(piece < C / 8 ? c_pages + row * C + piece * 8
+                                                                  : r_pages + row * R + (piece - C / 8) * 8);
+          }
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const int seg = threadIdx.x + (j0 + g) * THREADS;
+          if (j0 + g < KPT && seg < 32 * KSEG) {
+            const int key = seg / KSEG, piece = seg - key * KSEG;
+            *reinterpret_cast<bf16x8*>(Ks + key * KROW + piece * 8) = t[g];
+          }
+        }
+      }
+#pragma unroll
+      for (int j0 = 0; j0 < VPT; j0 += G) {
+        bf16x8 t[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          if (j0 + g < VPT) {
+            const int seg = threadIdx.x + (j0 + g) * THREADS;
+            const int u = seg / (C * 2), rem = seg - u * (C * 2), dim = rem >> 1, piece = rem & 1;
+            t[g] = *reinterpret_cast<const bf16x8*>(ct_pages + (row0[u] / page_size) * (size_t)page_size * C +
+                                                    (size_t)dim * page_size + row0[u] % page_size + piece * 8);
+          }
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          if (j0 + g < VPT) {
+            const int seg = threadIdx.x + (j0 + g) * THREADS;
+            const int u = seg / (C * 2), rem = seg - u * (C * 2), dim = rem >> 1, piece = rem & 1;
+            bf16x8 v = t[g];
+            const int k0 = base + u * 16 + piece * 8;
+            if (k0 + 7 > blk_hi) {
+#pragma unroll
+              for (int i = 0; i < 8; ++i)
+                if (k0 + i > blk_hi) v[i] = (__bf16)0.0f;
+            }
+            *reinterpret_cast<bf16x8*>(Vs + dim * LS_VROW + u * 16 + piece * 8) = v;
+          }
+        }
+      }
+    }
     __syncthreads();
+    if (AHEAD && base + 32 <= blk_hi) {
+      issue(base + 32);
+      if (base + 64 <= blk_hi) lookup(base + 64);
+    }
     if (!tile || base > key_hi || base + 31 < key_lo) continue;     // none of this block's keys is the tile's
     f32x4 s[2];
 #pragma unroll
