@@ -4,8 +4,9 @@ from .registry import (ConfigError, build_spec, config_class, config_from_dict, 
 from .spec import LayerSpec, ModelSpec, PartSpec, Run, layer
 from .qwen2 import Qwen2Config
 from .gemadra import GemadraConfig
+from .gidurax import GiduraxConfig
 from .presets import PRESETS, preset
 
 __all__ = ["EngineConfig", "ConfigError", "build_spec", "config_class", "config_from_dict",
            "known_architectures", "load_config", "register_architecture", "LayerSpec", "ModelSpec",
-           "PartSpec", "Run", "layer", "Qwen2Config", "GemadraConfig", "PRESETS", "preset"]
+           "PartSpec", "Run", "layer", "Qwen2Config", "GemadraConfig", "GiduraxConfig", "PRESETS", "preset"]

@@ -64,10 +64,13 @@ def layer(block: str, **parts: Optional[PartSpec]) -> LayerSpec:
 class Run:
     """One entry of the execution order.  ``layer`` indexes ``ModelSpec.layers`` (a layer may be
     named more than once: its weights are shared, each run has a cache of its own).  ``cache_of``
-    names an earlier run whose cache this run reads instead of keeping one itself."""
+    names an earlier run whose cache this run reads instead of keeping one itself.  ``opens_pass`` = t: the run is
+    the first of pass t over a stretch of layers that is walked several times, and the model's ``pass_entry`` part
+    is applied to the residual stream right before it."""
 
     layer: int
     cache_of: Optional[int] = None
+    opens_pass: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -81,8 +84,11 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     ignorable: Tuple[str, ...] = ()    # tensors a checkpoint may hold that no part of this model reads
+    pass_entry: Optional[PartSpec] = None   # what is done to the residual stream before a run with ``opens_pass``
 
     def __post_init__(self):
+        if self.pass_entry is None and any(run.opens_pass is not None for run in self.order):
+            raise ValueError("a run opens a pass, but the model has no pass_entry part")
         for i, run in enumerate(self.order):
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"order[{i}] names layer {run.layer}, but there are {len(self.layers)} layers")

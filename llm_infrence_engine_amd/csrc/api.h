@@ -6,7 +6,8 @@
 
 extern "C" {
 
-int ms_embed(const int* ids, const void* table, float* out, int n_tokens, int hidden, int dtype, hipStream_t stream);
+int ms_embed(const int* ids, const void* table, float* out, int n_tokens, int hidden, float scale, int dtype,
+             hipStream_t stream);
 
 int ms_rms_norm(float* x, const void* delta, int delta_dtype, int n_partials, long long partial_stride,
                 const float* weight, const int* rows, void* out, int n_rows, int hidden, float eps, int write_back,
@@ -105,8 +106,8 @@ int ms_paged_attention_generic(const void* q, long long q_stride, const void* k_
                                const int* block_table, int table_stride, const int* table_rows,
                                const int* n_live_tokens, const int* token_req, const int* positions,
                                void* out, long long out_stride, int n_tokens, int num_heads, int num_kv_heads,
-                               int head_dim, int page_size, long long num_pages, float scale, int window,
-                               int v_transposed, int dtype, hipStream_t stream);
+                               int head_dim, int value_dim, int page_size, long long num_pages, float scale, int window,
+                               int v_transposed, const float* sink, int dtype, hipStream_t stream);
 
 int ms_attention_mfma_supported(int head_dim, int page_size);
 
@@ -151,27 +152,30 @@ int ms_sample(const float* logits, long long ld, int n_rows, int vocab, const fl
 
 // ---- mixers with a fixed-size state (csrc/sequence.hip).  A step's requests: tokens q_start[r]..q_start[r+1]-1, state
 // slot state_slots[r]; token_req [n_tokens]; n_live_tokens (may be null): tokens from there on belong to no request.
-// Short causal convolution per channel: w float [channels, taps] (last column: the current token), state
+// Short causal convolution per channel: w float [channels, taps] (last column: the current token), bias float [channels]
+// or null, state
 // [slots, taps - 1, channels] in `dtype`.  mode 0: the sum, 1: x + the sum, 2: silu(the sum).  out must not be x.
 // With update_state the state becomes the last taps - 1 inputs of every request that has tokens (single_tokens: the
 // caller knows that no request has more than one token, and the same kernel moves the state on).
-int ms_short_conv(const void* x, long long x_stride, const float* w, void* state, const int* token_req,
+int ms_short_conv(const void* x, long long x_stride, const float* w, const float* bias, void* state, const int* token_req,
                   const int* q_start, const int* state_slots, const int* n_live_tokens, void* out, long long out_stride,
                   int n_tokens, int n_requests, int channels, int taps, int mode, int update_state, int single_tokens,
                   int dtype, hipStream_t stream);
 
-// Gated delta rule with a decay per head and key channel.  q, k [n, kv_heads * dim], v [n, heads * vdim], b [n, heads]
-// in `dtype` (rows qkv_stride / b_stride apart); a float [n, heads * dim] (the decay's input before dt_bias);
+// Gated delta rule.  q, k [n, kv_heads * dim], v [n, heads * vdim], b [n, heads] in `dtype` (rows qkv_stride / b_stride
+// apart); a: the decay's input before dt_bias, float [n, heads * dim] with dt_bias [heads * dim] (decay_per_channel: one
+// decay per head and key channel) or float [n, heads] with dt_bias [heads] (one decay per head);
 // state float [slots, heads, dim, vdim]; out float [n, heads * vdim].  single_tokens: the caller knows that no request
 // has more than one token (a decode step).
-int ms_gated_delta(const void* q, const void* k, const void* v, long long qkv_stride, const float* a, const void* b,
-                   long long b_stride, const float* A_log, const float* dt_bias, float* state, const int* q_start,
+int ms_gated_delta(const void* q, const void* k, const void* v, long long qkv_stride, const float* a,
+                   int decay_per_channel, const void* b, long long b_stride, const float* A_log, const float* dt_bias, float* state, const int* q_start,
                    const int* state_slots, float* out, int n_requests, int heads, int kv_heads, int dim, int vdim,
                    int single_tokens, int dtype, hipStream_t stream);
 
-// out[n, h, :] = o[n, h, :] / rms(o[n, h, :]) * weight * sigmoid(gate[n, h, :]); o float, gate and out in `dtype`.
+// out[n, h, :] = o[n, h, :] / rms(o[n, h, :]) * weight * act(gate[n, h, :]), act the sigmoid or (gate_silu) z * sigmoid(z);
+// o float, gate and out in `dtype`.
 int ms_gated_head_norm(const float* o, const float* weight, const void* gate, long long gate_stride, void* out,
-                       int n_tokens, int heads, int vdim, float eps, int dtype, hipStream_t stream);
+                       int n_tokens, int heads, int vdim, float eps, int gate_silu, int dtype, hipStream_t stream);
 
 // xIELU with pq = (p, q) on the device.
 int ms_xielu(const void* x, const float* pq, void* out, long long total, int dtype, hipStream_t stream);
@@ -201,5 +205,45 @@ int ms_latent_attention_mfma(const void* q, long long q_tok, long long q_head, c
                              const int* q_start, const int* context_lens, const float* sink, void* out, long long out_tok,
                              long long out_head, int n_requests, int max_q_len, int heads, int C, int R, int page_size,
                              long long num_pages, float scale, int window, hipStream_t stream);
+
+// ---- layers that normalise a sublayer's output before it joins the residual stream (csrc/residual_norm.hip)
+// x += w_post * rms_norm(y); then, if out is not null, out = w_next * rms_norm(x).  y [n, hidden] in y_dtype (rows y_stride
+// apart), x float [n, hidden], out in out_dtype.
+int ms_rms_norm_add(const void* y, long long y_stride, int y_dtype, const float* w_post, float eps_post, float* x,
+                    const float* w_next, float eps_next, void* out, int out_dtype, int n_rows, int hidden,
+                    hipStream_t stream);
+// x[n, :] += kept[n, :] (if not null) + vec[:] (if not null)
+int ms_add_rows(float* x, const float* kept, const float* vec, int n_rows, int hidden, hipStream_t stream);
+
+// ---- heads normalised instead of rotated (csrc/qk_norm.hip): RMS norm of every q and k head with q_weight / k_weight
+// [head_dim] (null: no norm), q times 1 + coef * ln(floor((p + 1) / every) + 1) (coef 0: none), k and v stored into pages
+// (null: not stored); qkv [n, nh * head_dim + nkv * head_dim + nkv * value_dim]
+int ms_qk_norm_store(void* qkv, long long stride, const float* q_weight, const float* k_weight, float eps,
+                     const int* positions, float coef, int every, const int* slots, void* k_pages, void* v_pages,
+                     int n_tokens, int num_heads, int num_kv_heads, int head_dim, int value_dim, int page_size,
+                     int v_transposed, int dtype, hipStream_t stream);
+
+// ---- the selective scan of a state-space mixer (csrc/scan.hip)
+int ms_selective_scan(const void* x, long long x_stride, const float* dt_in, const float* dt_bias, const float* A,
+                      const void* B, const void* C, long long bc_stride, const float* D, const void* z, long long z_stride,
+                      float* state, const int* q_start, const int* state_slots, void* out, long long out_stride,
+                      int n_requests, int channels, int states, int dtype, hipStream_t stream);
+
+// ---- routed experts (csrc/experts.hip)
+int ms_gelu(const void* x, void* out, long long total, int dtype, hipStream_t stream);
+// softmax over logits[n, :n_out] (rows ld apart), the `top` largest of score + correction: ids / weights [n, top]
+int ms_moe_route(const float* logits, long long ld, const float* correction, int n_tokens, int n_out, int top, int* ids,
+                 float* weights, hipStream_t stream);
+int ms_moe_tile_rows();
+// rows [tiles * ms_moe_tile_rows()] and tile_expert [tiles] from ids [n_items]; ids >= n_experts take no row
+int ms_moe_align(const int* ids, int n_items, int n_experts, int tiles, int* rows, int* tile_expert, hipStream_t stream);
+// for every tile t with an expert e and each of its rows i (flat position p = t * tile + i, item = rows[p] >= 0):
+// out[out_scatter ? item : p] = act(w[e] . in[in_div ? item / in_div : p]); w [experts, n_out, K]
+int ms_grouped_gemm(const void* in, long long in_stride, const void* w, const int* rows, const int* tile_expert, void* out,
+                    long long out_stride, int tiles, int n_out, int K, int in_div, int out_scatter, int act, int dtype,
+                    int out_dtype, hipStream_t stream);
+int ms_moe_combine(const float* part, const int* ids, const float* weights, const void* h, long long h_stride,
+                   const void* shared, int shared_dtype, const float* gate, long long gate_stride, float* out,
+                   int n_tokens, int top, int n_experts, int hidden, int dtype, hipStream_t stream);
 
 }  // extern "C"

@@ -1,5 +1,6 @@
-// Paged causal attention with grouped heads, any head size that is a multiple of 4 up to 256, for any mix
-// of prompt portions and single decoded tokens.  One wave per (token, query head): scores, running
+// Paged causal attention with grouped heads, any key size that is a multiple of 4 up to 256 and any value size up
+// to 256, for any mix of prompt portions and single decoded tokens.  `sink` (may be null): one number per query
+// head whose exponential joins the softmax's denominator; it has no key and no value.  One wave per (token, query head): scores, running
 // maximum, exponentials, their sum and the weighted sum of values are all float.  It reads keys and
 // values in place through the request's block table and never reads a key beyond the token's own
 // position, so what a reused page still holds from an earlier request cannot reach the result.
@@ -20,8 +21,9 @@ paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T
                                const T* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
                                const int* __restrict__ table_rows, const int* __restrict__ n_live_tokens,
                                const int* __restrict__ token_req, const int* __restrict__ positions,
-                               T* __restrict__ out, size_t out_stride, int n_tokens, int nh, int nkv, int d,
-                               int page_size, float scale, int window, int v_transposed) {
+                               T* __restrict__ out, size_t out_stride, int n_tokens, int nh, int nkv, int d, int dv,
+                               int page_size, float scale, int window, int v_transposed,
+                               const float* __restrict__ sink) {
   __shared__ float qs[WAVES][MAX_D];
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const long long item = (long long)blockIdx.x * WAVES + wave;
@@ -77,22 +79,23 @@ paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T
       const float pj = __shfl(p, jj, MS_WAVE);
       const int vrow = __shfl(row, jj, MS_WAVE);
       // value pages are [page][kv head][slot][dim], or transposed [page][kv head][dim][slot]
-      const T* vp = v_transposed ? v_pages + (size_t)(vrow / page_size) * page_size * d + vrow % page_size
-                                 : v_pages + (size_t)vrow * d;
+      const T* vp = v_transposed ? v_pages + (size_t)(vrow / page_size) * page_size * dv + vrow % page_size
+                                 : v_pages + (size_t)vrow * dv;
       const int vs = v_transposed ? page_size : 1;
 #pragma unroll
       for (int c = 0; c < MAX_D / MS_WAVE; ++c) {
         const int i = lane + c * MS_WAVE;
-        if (i < d) acc[c] = fmaf(pj, to_float(vp[(size_t)i * vs]), acc[c]);
+        if (i < dv) acc[c] = fmaf(pj, to_float(vp[(size_t)i * vs]), acc[c]);
       }
     }
   }
-  T* op = out + (size_t)n * out_stride + (size_t)h * d;
+  T* op = out + (size_t)n * out_stride + (size_t)h * dv;
+  if (sink) l += expf(sink[h] - m);   // m is finite: a token always sees its own key
   const float inv = 1.0f / l;
 #pragma unroll
   for (int c = 0; c < MAX_D / MS_WAVE; ++c) {
     const int i = lane + c * MS_WAVE;
-    if (i < d) op[i] = from_float<T>(acc[c] * inv);
+    if (i < dv) op[i] = from_float<T>(acc[c] * inv);
   }
 }
 
@@ -102,17 +105,17 @@ extern "C" int ms_paged_attention_generic(const void* q, long long q_stride, con
                                           const int* block_table, int table_stride, const int* table_rows,
                                           const int* n_live_tokens, const int* token_req,
                                           const int* positions, void* out, long long out_stride, int n_tokens,
-                                          int num_heads, int num_kv_heads, int head_dim, int page_size,
+                                          int num_heads, int num_kv_heads, int head_dim, int value_dim, int page_size,
                                           long long num_pages, float scale, int window, int v_transposed,
-                                          int dtype, hipStream_t stream) {
+                                          const float* sink, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || page_size <= 0 || table_stride <= 0)
     return MS_BAD_ARG;
-  if (head_dim <= 0 || head_dim % 4 || head_dim > MAX_D) return MS_UNSUPPORTED;
+  if (head_dim <= 0 || head_dim % 4 || head_dim > MAX_D || value_dim <= 0 || value_dim > MAX_D) return MS_UNSUPPORTED;
   if (num_pages * num_kv_heads * page_size >= (1ll << 31)) return MS_UNSUPPORTED;  // row index is an int
   const long long items = (long long)n_tokens * num_heads;
   dim3 grid((unsigned)((items + WAVES - 1) / WAVES)), block(WAVES * MS_WAVE);
-#define LAUNCH(T) paged_attention_generic_kernel<T><<<grid, block, 0, stream>>>((const T*)q, (size_t)q_stride, (const T*)k_pages, (const T*)v_pages, block_table, table_stride, table_rows, n_live_tokens, token_req, positions, (T*)out, (size_t)out_stride, n_tokens, num_heads, num_kv_heads, head_dim, page_size, scale, window, v_transposed)
+#define LAUNCH(T) paged_attention_generic_kernel<T><<<grid, block, 0, stream>>>((const T*)q, (size_t)q_stride, (const T*)k_pages, (const T*)v_pages, block_table, table_stride, table_rows, n_live_tokens, token_req, positions, (T*)out, (size_t)out_stride, n_tokens, num_heads, num_kv_heads, head_dim, value_dim, page_size, scale, window, v_transposed, sink)
   if (dtype == MS_F32) LAUNCH(float);
   else if (dtype == MS_BF16) LAUNCH(bf16);
   else return MS_BAD_ARG;

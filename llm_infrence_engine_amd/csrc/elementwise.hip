@@ -7,22 +7,23 @@
 #include <algorithm>
 
 // ------------------------------------------------------------------------------------------------
-// out[n, :] = float(table[ids[n], :])
+// out[n, :] = float(table[ids[n], :]) * scale
 template <typename T>
-__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int H) {
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int H,
+                             float scale) {
   const int n = blockIdx.x;
   const T* row = table + (size_t)ids[n] * H;
   float* o = out + (size_t)n * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_float(row[i]);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_float(row[i]) * scale;
 }
 
-extern "C" int ms_embed(const int* ids, const void* table, float* out, int n_tokens, int hidden, int dtype,
+extern "C" int ms_embed(const int* ids, const void* table, float* out, int n_tokens, int hidden, float scale, int dtype,
                         hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
   if (hidden <= 0) return MS_BAD_ARG;
   dim3 grid(n_tokens), block(256);
-  if (dtype == MS_F32) embed_kernel<float><<<grid, block, 0, stream>>>(ids, (const float*)table, out, hidden);
-  else if (dtype == MS_BF16) embed_kernel<bf16><<<grid, block, 0, stream>>>(ids, (const bf16*)table, out, hidden);
+  if (dtype == MS_F32) embed_kernel<float><<<grid, block, 0, stream>>>(ids, (const float*)table, out, hidden, scale);
+  else if (dtype == MS_BF16) embed_kernel<bf16><<<grid, block, 0, stream>>>(ids, (const bf16*)table, out, hidden, scale);
   else return MS_BAD_ARG;
   return ms_launch_status();
 }

@@ -1,0 +1,268 @@
+// Kernels of a feed-forward made of routed experts, all driven by device data so that a step can be captured:
+//   route    per token: softmax over the router's outputs, the `top` largest of (score + correction), their scores
+//   align    rows (token, choice) grouped by expert into tiles of TILE rows, each tile of one expert
+//   grouped  out[row] = act(W[expert of the row's tile] . in[row]) for every tile, gathered / scattered by the rows' list
+//   combine  out[n] = sum_j weight[n, j] * (expert j's row, or the token's input for an identity expert)
+//                     (+ sigmoid(gate[n]) * shared[n])
+// and the exact gelu, z/2 (1 + erf(z / sqrt 2)).  Router scores, weights and all sums are float.
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+constexpr int ROUTE_MAX_PER_LANE = 16;     // router outputs a lane holds: up to 1024 outputs
+constexpr int ROUTE_MAX_TOP = 32;
+
+__device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f)); }
+
+template <typename T>
+__global__ void gelu_kernel(const T* __restrict__ x, T* __restrict__ out, size_t total) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride)
+    out[i] = from_float<T>(gelu_erf(to_float(x[i])));
+}
+
+// One wave per token.  Ties go to the lower index.
+__global__ void __launch_bounds__(256)
+moe_route_kernel(const float* __restrict__ logits, size_t ld, const float* __restrict__ correction, int n_tokens,
+                 int n_out, int top, int* __restrict__ ids, float* __restrict__ weights) {
+  const int lane = threadIdx.x & (MS_WAVE - 1);
+  const int n = blockIdx.x * (blockDim.x / MS_WAVE) + threadIdx.x / MS_WAVE;
+  if (n >= n_tokens) return;
+  const float* z = logits + (size_t)n * ld;
+  float s[ROUTE_MAX_PER_LANE], c[ROUTE_MAX_PER_LANE];
+  float big = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < ROUTE_MAX_PER_LANE; ++i) {
+    const int e = lane + i * MS_WAVE;
+    s[i] = e < n_out ? z[e] : -INFINITY;
+    big = fmaxf(big, s[i]);
+  }
+  big = wave_max(big);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < ROUTE_MAX_PER_LANE; ++i) {
+    const int e = lane + i * MS_WAVE;
+    s[i] = e < n_out ? expf(s[i] - big) : 0.f;
+    sum += s[i];
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.0f / sum;
+#pragma unroll
+  for (int i = 0; i < ROUTE_MAX_PER_LANE; ++i) {
+    const int e = lane + i * MS_WAVE;
+    s[i] *= inv;
+    c[i] = e < n_out ? s[i] + (correction ? correction[e] : 0.f) : -INFINITY;
+  }
+  for (int j = 0; j < top; ++j) {
+    float bv = -INFINITY, bs = 0.f;
+    int be = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < ROUTE_MAX_PER_LANE; ++i) {
+      const int e = lane + i * MS_WAVE;
+      if (c[i] > bv) { bv = c[i]; be = e; bs = s[i]; }   // a lane's indices rise with i: the first maximum stays
+    }
+#pragma unroll
+    for (int o = MS_WAVE / 2; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, MS_WAVE), os = __shfl_xor(bs, o, MS_WAVE);
+      const int oe = __shfl_xor(be, o, MS_WAVE);
+      if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; bs = os; }
+    }
+    if (lane == 0) { ids[(size_t)n * top + j] = be; weights[(size_t)n * top + j] = bs; }
+#pragma unroll
+    for (int i = 0; i < ROUTE_MAX_PER_LANE; ++i)
+      if (lane + i * MS_WAVE == be) c[i] = -INFINITY;
+  }
+}
+
+// One block.  rows[cap] (cap = tiles * tile): for every tile its rows' flat index n * top + j, or -1; tile_expert[tiles]:
+// the tile's expert, or -1 for a tile nobody uses.  Choices of experts >= n_experts (identities) take no row.
+__global__ void __launch_bounds__(1024)
+moe_align_kernel(const int* __restrict__ ids, int n_items, int n_experts, int tile, int tiles, int* __restrict__ rows,
+                 int* __restrict__ tile_expert) {
+  extern __shared__ int sh[];     // counts [n_experts], first row of each expert [n_experts + 1]
+  int* count = sh;
+  int* first = sh + n_experts;
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count[e] = 0;
+  for (int i = threadIdx.x; i < tiles * tile; i += blockDim.x) rows[i] = -1;
+  for (int t = threadIdx.x; t < tiles; t += blockDim.x) tile_expert[t] = -1;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_items; i += blockDim.x) {
+    const int e = ids[i];
+    if (e >= 0 && e < n_experts) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      first[e] = at;
+      at += (count[e] + tile - 1) / tile * tile;
+    }
+    first[n_experts] = at;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+    for (int t = first[e] / tile; t < first[e + 1] / tile; ++t) tile_expert[t] = e;
+    count[e] = 0;       // now the cursor within the expert's rows
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_items; i += blockDim.x) {
+    const int e = ids[i];
+    if (e >= 0 && e < n_experts) rows[first[e] + atomicAdd(&count[e], 1)] = i;
+  }
+}
+
+// Vector-ALU product of every tile with its expert's matrix: float accumulation in the order of k, whatever the
+// batch.  A block owns GM rows of a tile by GN output features; K walks in steps of GK through LDS.
+constexpr int GM = 16, GN = 64, GK = 32;
+
+template <typename T, typename TO>
+__global__ void __launch_bounds__(256)
+grouped_gemm_kernel(const T* __restrict__ in, size_t in_stride, const T* __restrict__ w, const int* __restrict__ rows,
+                    const int* __restrict__ tile_expert, TO* __restrict__ out, size_t out_stride, int n_out, int K,
+                    int in_div, int out_scatter, int act) {
+  __shared__ float As[GM][GK + 1], Ws[GN][GK + 1];
+  __shared__ int s_row[GM];
+  const int tile = blockIdx.x;
+  const int e = tile_expert[tile];
+  if (e < 0) return;
+  const int n0 = blockIdx.y * GN;
+  const int tid = threadIdx.x;
+  if (tid < GM) s_row[tid] = rows[tile * GM + tid];
+  __syncthreads();
+  const T* we = w + (size_t)e * n_out * K;
+  const int r = tid / 16, cg = tid % 16;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += GK) {
+    for (int i = tid; i < GM * GK; i += 256) {
+      const int rr = i / GK, kk = i % GK;
+      const int item = s_row[rr];
+      float v = 0.f;
+      if (item >= 0 && k0 + kk < K) {
+        const size_t src = in_div > 0 ? (size_t)(item / in_div) : (size_t)(tile * GM + rr);
+        v = to_float(in[src * in_stride + k0 + kk]);
+      }
+      As[rr][kk] = v;
+    }
+    for (int i = tid; i < GN * GK; i += 256) {
+      const int cc = i / GK, kk = i % GK;
+      Ws[cc][kk] = (n0 + cc < n_out && k0 + kk < K) ? to_float(we[(size_t)(n0 + cc) * K + k0 + kk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < GK; ++kk) {
+      const float a = As[r][kk];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = fmaf(a, Ws[cg + 16 * j][kk], acc[j]);
+    }
+    __syncthreads();
+  }
+  const int item = s_row[r];
+  if (item < 0) return;
+  const size_t dst = out_scatter ? (size_t)item : (size_t)(tile * GM + r);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = n0 + cg + 16 * j;
+    if (c < n_out) out[dst * out_stride + c] = from_float<TO>(act ? gelu_erf(acc[j]) : acc[j]);
+  }
+}
+
+// out[n, :] = sum_j weights[n, j] * (ids[n, j] < n_experts ? part[n * top + j, :] : h[n, :]) + sigmoid(gate[n]) * shared[n, :]
+template <typename T, typename TS>
+__global__ void __launch_bounds__(256)
+moe_combine_kernel(const float* __restrict__ part, const int* __restrict__ ids, const float* __restrict__ weights,
+                   const T* __restrict__ h, size_t h_stride, const TS* __restrict__ shared, const float* __restrict__ gate,
+                   size_t gate_stride, float* __restrict__ out, int top, int n_experts, int H) {
+  const int n = blockIdx.x;
+  __shared__ int s_id[ROUTE_MAX_TOP];
+  __shared__ float s_w[ROUTE_MAX_TOP];
+  if ((int)threadIdx.x < top) {
+    s_id[threadIdx.x] = ids[(size_t)n * top + threadIdx.x];
+    s_w[threadIdx.x] = weights[(size_t)n * top + threadIdx.x];
+  }
+  __syncthreads();
+  float g = 0.f;
+  if (shared) { const float z = gate[(size_t)n * gate_stride]; g = 1.0f / (1.0f + expf(-z)); }
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < top; ++j) {
+      const float v = s_id[j] < n_experts ? part[((size_t)n * top + j) * H + i] : to_float(h[(size_t)n * h_stride + i]);
+      acc = fmaf(s_w[j], v, acc);
+    }
+    if (shared) acc = fmaf(g, to_float(shared[(size_t)n * H + i]), acc);
+    out[(size_t)n * H + i] = acc;
+  }
+}
+
+}  // namespace
+
+extern "C" int ms_gelu(const void* x, void* out, long long total, int dtype, hipStream_t stream) {
+  if (total <= 0) return MS_OK;
+  int blocks = (int)((total + 1023) / 1024);
+  if (blocks > 8192) blocks = 8192;
+  if (dtype == MS_F32) gelu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)x, (float*)out, (size_t)total);
+  else if (dtype == MS_BF16) gelu_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)x, (bf16*)out, (size_t)total);
+  else return MS_BAD_ARG;
+  return ms_launch_status();
+}
+
+extern "C" int ms_moe_route(const float* logits, long long ld, const float* correction, int n_tokens, int n_out, int top,
+                            int* ids, float* weights, hipStream_t stream) {
+  if (n_tokens <= 0) return MS_OK;
+  if (n_out <= 0 || top <= 0 || top > n_out) return MS_BAD_ARG;
+  if (n_out > ROUTE_MAX_PER_LANE * MS_WAVE || top > ROUTE_MAX_TOP) return MS_UNSUPPORTED;
+  moe_route_kernel<<<(n_tokens + 3) / 4, 256, 0, stream>>>(logits, (size_t)ld, correction, n_tokens, n_out, top, ids,
+                                                           weights);
+  return ms_launch_status();
+}
+
+extern "C" int ms_moe_tile_rows() { return GM; }
+
+extern "C" int ms_moe_align(const int* ids, int n_items, int n_experts, int tiles, int* rows, int* tile_expert,
+                            hipStream_t stream) {
+  if (n_items <= 0 || tiles <= 0) return MS_OK;
+  if (n_experts <= 0) return MS_BAD_ARG;
+  if (n_experts > 4096) return MS_UNSUPPORTED;
+  if ((long long)tiles * GM < (long long)n_items + (long long)n_experts * (GM - 1)) return MS_BAD_ARG;
+  moe_align_kernel<<<1, 1024, (2 * n_experts + 1) * sizeof(int), stream>>>(ids, n_items, n_experts, GM, tiles, rows,
+                                                                          tile_expert);
+  return ms_launch_status();
+}
+
+extern "C" int ms_grouped_gemm(const void* in, long long in_stride, const void* w, const int* rows, const int* tile_expert,
+                               void* out, long long out_stride, int tiles, int n_out, int K, int in_div, int out_scatter,
+                               int act, int dtype, int out_dtype, hipStream_t stream) {
+  if (tiles <= 0) return MS_OK;
+  if (n_out <= 0 || K <= 0 || in_div < 0) return MS_BAD_ARG;
+  const int cb = (n_out + GN - 1) / GN;
+  if (cb > 65535) return MS_UNSUPPORTED;
+  dim3 grid(tiles, cb), block(256);
+#define LAUNCH(T, TO)                                                                                                 \
+  grouped_gemm_kernel<T, TO><<<grid, block, 0, stream>>>((const T*)in, (size_t)in_stride, (const T*)w, rows,          \
+                                                         tile_expert, (TO*)out, (size_t)out_stride, n_out, K, in_div, \
+                                                         out_scatter, act)
+  if (dtype == MS_F32 && out_dtype == MS_F32) LAUNCH(float, float);
+  else if (dtype == MS_BF16 && out_dtype == MS_F32) LAUNCH(bf16, float);
+  else if (dtype == MS_BF16 && out_dtype == MS_BF16) LAUNCH(bf16, bf16);
+  else return MS_BAD_ARG;
+#undef LAUNCH
+  return ms_launch_status();
+}
+
+extern "C" int ms_moe_combine(const float* part, const int* ids, const float* weights, const void* h, long long h_stride,
+                              const void* shared, int shared_dtype, const float* gate, long long gate_stride, float* out,
+                              int n_tokens, int top, int n_experts, int hidden, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return MS_OK;
+  if (top <= 0 || top > ROUTE_MAX_TOP || hidden <= 0 || (shared != nullptr && gate == nullptr)) return MS_BAD_ARG;
+  dim3 grid(n_tokens), block(256);
+#define LAUNCH(T, TS)                                                                                                \
+  moe_combine_kernel<T, TS><<<grid, block, 0, stream>>>(part, ids, weights, (const T*)h, (size_t)h_stride,           \
+                                                        (const TS*)shared, gate, (size_t)gate_stride, out, top,      \
+                                                        n_experts, hidden)
+  if (dtype == MS_F32) LAUNCH(float, float);
+  else if (dtype == MS_BF16 && shared_dtype == MS_F32) LAUNCH(bf16, float);
+  else if (dtype == MS_BF16) LAUNCH(bf16, bf16);
+  else return MS_BAD_ARG;
+#undef LAUNCH
+  return ms_launch_status();
+}

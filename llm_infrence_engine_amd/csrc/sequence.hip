@@ -17,10 +17,10 @@ __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf
 // ------------------------------------------------------------------------------------------------
 // y[n, c] = act(sum_j w[c, j] * in(t - taps + 1 + j)) (+ x[n, c]), t the token's index within its portion;
 // in(i) is the portion's own input for i >= 0 and the state (the taps - 1 inputs before the portion) for i < 0.
-// mode 0: the sum; 1: x + the sum; 2: silu of the sum.
+// mode 0: the sum; 1: x + the sum; 2: silu of the sum.  `bias` (may be null): one number per channel, added to the sum.
 template <typename T>
 __global__ void short_conv_kernel(const T* __restrict__ x, size_t x_stride, const float* __restrict__ w,
-                                  const T* state, const int* __restrict__ token_req,
+                                  const float* __restrict__ bias, const T* state, const int* __restrict__ token_req,
                                   const int* __restrict__ q_start, const int* __restrict__ state_slots,
                                   const int* __restrict__ n_live_tokens, T* __restrict__ out, size_t out_stride,
                                   int C, int taps, int mode, T* state_out) {
@@ -32,7 +32,7 @@ __global__ void short_conv_kernel(const T* __restrict__ x, size_t x_stride, cons
   const int s = q_start[r];
   const int t = n - s;
   const T* st = state + (size_t)state_slots[r] * (taps - 1) * C;
-  float acc = 0.f;
+  float acc = bias ? bias[c] : 0.f;
   for (int j = 0; j < taps; ++j) {
     const int i = t - taps + 1 + j;
     const float v = i >= 0 ? to_float(x[(size_t)(s + i) * x_stride + c]) : to_float(st[(size_t)(taps - 1 + i) * C + c]);
@@ -111,7 +111,7 @@ constexpr int DELTA_CHUNK = 16;
 template <typename T, int DPT, int LPC, bool SINGLE, bool SPLIT>
 __global__ void __launch_bounds__(SPLIT ? 512 : 256, SINGLE ? 3 : 1)
 gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, size_t qkv_stride,
-                   const float* __restrict__ a, const T* __restrict__ b, size_t b_stride,
+                   const float* __restrict__ a, int decay_per_channel, const T* __restrict__ b, size_t b_stride,
                    const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ state,
                    const int* __restrict__ q_start, const int* __restrict__ state_slots, float* __restrict__ out,
                    int H, int G, int D, int E, int cols_per_block, int chunk) {
@@ -160,12 +160,17 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
       const size_t n = (size_t)(s0 + c0 + tl);
       const T* qp = q + n * qkv_stride + (size_t)kvh * D;
       const T* kp = k + n * qkv_stride + (size_t)kvh * D;
-      const float* ap = a + n * (size_t)H * D + (size_t)h * D;
+      // the decay's input: one number per head and key channel, or one per head that all its channels share
+      const float* ap = decay_per_channel ? a + n * (size_t)H * D + (size_t)h * D : a + n * (size_t)H + h;
 #pragma unroll
       for (int e = 0; e < EPL; ++e) {
         const int i = l16 + e * LT;
         const bool in = i < D;
-        if (in) { qr[e] = qp[i]; kr[e] = kp[i]; ar[e] = ap[i]; dr[e] = dt_bias[(size_t)h * D + i]; }
+        if (in) {
+          qr[e] = qp[i]; kr[e] = kp[i];
+          ar[e] = ap[decay_per_channel ? i : 0];
+          dr[e] = dt_bias[decay_per_channel ? (size_t)h * D + i : (size_t)h];
+        }
       }
       if (l16 == 0) br = b[n * b_stride + h];
     }
@@ -323,11 +328,12 @@ gated_delta_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __
 }
 
 // ------------------------------------------------------------------------------------------------
-// y[n, h, :] = o[n, h, :] / sqrt(mean(o[n, h, :]^2) + eps) * w[:] * sigmoid(gate[n, h, :]); one wave per (token, head).
+// y[n, h, :] = o[n, h, :] / sqrt(mean(o[n, h, :]^2) + eps) * w[:] * act(gate[n, h, :]), act the sigmoid (gate_silu 0) or
+// z * sigmoid(z) (1); one wave per (token, head).
 template <typename T>
 __global__ void gated_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ w,
                                        const T* __restrict__ gate, size_t gate_stride, T* __restrict__ out,
-                                       long long items, int H, int E, float eps) {
+                                       long long items, int H, int E, float eps, int gate_silu) {
   const int lane = threadIdx.x & (MS_WAVE - 1);
   const long long item = (long long)blockIdx.x * (blockDim.x / MS_WAVE) + threadIdx.x / MS_WAVE;
   if (item >= items) return;
@@ -340,8 +346,10 @@ __global__ void gated_head_norm_kernel(const float* __restrict__ o, const float*
   const float inv = 1.0f / sqrtf(ss / (float)E + eps);
   const T* gp = gate + (size_t)n * gate_stride + (size_t)h * E;
   T* yp = out + (size_t)item * E;
-  for (int i = lane; i < E; i += MS_WAVE)
-    yp[i] = from_float<T>(op[i] * inv * w[i] * sigmoid_f(to_float(gp[i])));
+  for (int i = lane; i < E; i += MS_WAVE) {
+    const float z = to_float(gp[i]);
+    yp[i] = from_float<T>(op[i] * inv * w[i] * (gate_silu ? z * sigmoid_f(z) : sigmoid_f(z)));
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -371,7 +379,8 @@ __global__ void xielu_kernel(const T* __restrict__ x, const float* __restrict__ 
 
 }  // namespace
 
-extern "C" int ms_short_conv(const void* x, long long x_stride, const float* w, void* state, const int* token_req,
+extern "C" int ms_short_conv(const void* x, long long x_stride, const float* w, const float* bias, void* state,
+                             const int* token_req,
                              const int* q_start, const int* state_slots, const int* n_live_tokens, void* out,
                              long long out_stride, int n_tokens, int n_requests, int channels, int taps, int mode,
                              int update_state, int single_tokens, int dtype, hipStream_t stream) {
@@ -385,7 +394,7 @@ extern "C" int ms_short_conv(const void* x, long long x_stride, const float* w, 
 #define LAUNCH(T)                                                                                                       \
   do {                                                                                                                  \
     const bool fused = update_state && single_tokens && taps > 1;                                                       \
-    short_conv_kernel<T><<<grid, block, 0, stream>>>((const T*)x, (size_t)x_stride, w, (const T*)state, token_req,     \
+    short_conv_kernel<T><<<grid, block, 0, stream>>>((const T*)x, (size_t)x_stride, w, bias, (const T*)state, token_req, \
                                                      q_start, state_slots, n_live_tokens, (T*)out, (size_t)out_stride, \
                                                      channels, taps, mode, fused ? (T*)state : nullptr);               \
     if (update_state && taps > 1 && !fused)                                                                             \
@@ -400,7 +409,7 @@ extern "C" int ms_short_conv(const void* x, long long x_stride, const float* w, 
 }
 
 extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long long qkv_stride, const float* a,
-                              const void* b, long long b_stride, const float* A_log, const float* dt_bias,
+                              int decay_per_channel, const void* b, long long b_stride, const float* A_log, const float* dt_bias,
                               float* state, const int* q_start, const int* state_slots, float* out, int n_requests,
                               int heads, int kv_heads, int dim, int vdim, int single_tokens, int dtype,
                               hipStream_t stream) {
@@ -429,7 +438,8 @@ extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long 
   if (lds > 65536) return MS_UNSUPPORTED;
 #define LAUNCH1(T, DPT, LPC, ONE, TWO)                                                                                  \
   gated_delta_kernel<T, DPT, LPC, ONE, TWO><<<grid, dim3(threads * ((TWO) ? 2 : 1)), lds * ((TWO) ? 2 : 1), stream>>>(  \
-      (const T*)q, (const T*)k, (const T*)v, (size_t)qkv_stride, a, (const T*)b, (size_t)b_stride, A_log, dt_bias,     \
+      (const T*)q, (const T*)k, (const T*)v, (size_t)qkv_stride, a, decay_per_channel, (const T*)b, (size_t)b_stride,  \
+      A_log, dt_bias,                                                                                                   \
       state, q_start, state_slots, out, heads, kv_heads, dim, vdim, cols, chunk)
 #define LAUNCH(T, DPT, LPC)                                                                                             \
   do {                                                                                                                  \
@@ -457,7 +467,7 @@ extern "C" int ms_gated_delta(const void* q, const void* k, const void* v, long 
 }
 
 extern "C" int ms_gated_head_norm(const float* o, const float* weight, const void* gate, long long gate_stride,
-                                  void* out, int n_tokens, int heads, int vdim, float eps, int dtype,
+                                  void* out, int n_tokens, int heads, int vdim, float eps, int gate_silu, int dtype,
                                   hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
   if (heads <= 0 || vdim <= 0) return MS_BAD_ARG;
@@ -466,10 +476,10 @@ extern "C" int ms_gated_head_norm(const float* o, const float* weight, const voi
   dim3 grid((unsigned)((items + waves - 1) / waves)), block(waves * MS_WAVE);
   if (dtype == MS_F32)
     gated_head_norm_kernel<float><<<grid, block, 0, stream>>>(o, weight, (const float*)gate, (size_t)gate_stride,
-                                                              (float*)out, items, heads, vdim, eps);
+                                                              (float*)out, items, heads, vdim, eps, gate_silu);
   else if (dtype == MS_BF16)
     gated_head_norm_kernel<bf16><<<grid, block, 0, stream>>>(o, weight, (const bf16*)gate, (size_t)gate_stride,
-                                                             (bf16*)out, items, heads, vdim, eps);
+                                                             (bf16*)out, items, heads, vdim, eps, gate_silu);
   else return MS_BAD_ARG;
   return ms_launch_status();
 }

@@ -20,7 +20,7 @@ _CODES = {1: "bad argument", 2: "unsupported size", 3: "launch failed"}
 _c_int, _c_ll, _c_float, _c_ptr = ctypes.c_int, ctypes.c_longlong, ctypes.c_float, ctypes.c_void_p
 
 _SIGNATURES = {
-    "ms_embed": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_embed": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "ms_rms_norm": [_c_ptr, _c_ptr, _c_int, _c_int, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int,
                     _c_int, _c_ptr],
     "ms_rms_norm_pair": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
@@ -61,8 +61,8 @@ _SIGNATURES = {
     "ms_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ll, _c_ll, _c_ll, _c_int,
                         _c_int, _c_int, _c_ptr],
     "ms_paged_attention_generic": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                                   _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float, _c_int, _c_int,
-                                   _c_int, _c_ptr],
+                                   _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float, _c_int, _c_int,
+                                   _c_ptr, _c_int, _c_ptr],
     "ms_attention_mfma_supported": [_c_int, _c_int],
     "ms_paged_attention_mfma": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll,
                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
@@ -73,11 +73,11 @@ _SIGNATURES = {
     "ms_sample": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                   _c_ptr],
     "ms_sample_workspace_bytes": [_c_int],
-    "ms_short_conv": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int,
-                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
-    "ms_gated_delta": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
-    "ms_gated_head_norm": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "ms_short_conv": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int,
+                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_gated_delta": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_int, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                       _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_gated_head_norm": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "ms_xielu": [_c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_head_matmul": [_c_ptr, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_ll, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int,
                        _c_int, _c_int, _c_ptr],
@@ -92,6 +92,21 @@ _SIGNATURES = {
     "ms_latent_attention": [_c_ptr, _c_ll, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                             _c_ptr, _c_ll, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float, _c_int, _c_int,
                             _c_ptr],
+    "ms_rms_norm_add": [_c_ptr, _c_ll, _c_int, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_int, _c_int, _c_int,
+                        _c_ptr],
+    "ms_add_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "ms_qk_norm_store": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_float, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_selective_scan": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_ptr,
+                          _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_gelu": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
+    "ms_moe_route": [_c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
+    "ms_moe_tile_rows": [],
+    "ms_moe_align": [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
+    "ms_grouped_gemm": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                        _c_int, _c_int, _c_ptr],
+    "ms_moe_combine": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_int, _c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int,
+                       _c_int, _c_int, _c_ptr],
 }
 
 _fn = {}
@@ -180,13 +195,14 @@ def _ptr(t: Optional[torch.Tensor]):
 
 
 # ------------------------------------------------------------------------------------------------
-def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[n] = float(table[ids[n]]).  ids int32 [N] (checked against the table by the caller), out float32 [N, H]."""
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[n] = float(table[ids[n]]) * scale.  ids int32 [N] (checked against the table by the caller), out float32 [N, H]."""
     _check(ids, "ids", torch.int32)
     _check(table, "table")
     V, H = table.shape
     _check(out, "out", torch.float32, (ids.numel(), H))
-    _call("ms_embed", ids.data_ptr(), table.data_ptr(), out.data_ptr(), ids.numel(), H, _code(table.dtype), _stream())
+    _call("ms_embed", ids.data_ptr(), table.data_ptr(), out.data_ptr(), ids.numel(), H, float(scale), _code(table.dtype),
+          _stream())
     return out
 
 
@@ -355,8 +371,9 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def _v_shape(k_pages: torch.Tensor, v_transposed: bool):
+def _v_shape(k_pages: torch.Tensor, v_transposed: bool, value_dim: Optional[int] = None):
     P, nkv, page_size, d = k_pages.shape
+    d = d if value_dim is None else value_dim
     return (P, nkv, d, page_size) if v_transposed else (P, nkv, page_size, d)
 
 
@@ -701,7 +718,7 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
                             token_req: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, num_heads: int,
                             scale: float, window: Optional[int] = None, v_transposed: bool = False,
                             table_rows: Optional[torch.Tensor] = None,
-                            n_live_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
+                            n_live_tokens: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[n, h] = softmax(scale * q[n, h] . K[keys visible to n]) V, keys read in place from pages.
 
     q: [N, >= nh * d] (a row slice of the fused projection is fine), out [N, nh * d],
@@ -709,15 +726,21 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     [rows, max_pages], token_req / positions int32 [N].
     Token n sees keys 0..positions[n] of request token_req[n] (the last ``window`` of them if given), whose
     pages are row ``table_rows[token_req[n]]`` of the table (row token_req[n] without ``table_rows``).  With
-    ``n_live_tokens`` (a device int) tokens from that index on are left alone."""
+    ``n_live_tokens`` (a device int) tokens from that index on are left alone.  Values may have another size than
+    keys (the value pages say which; out is then [N, nh * that size]).  ``sink`` float [nh]: exp(sink[h]) joins the
+    denominator of head h's softmax."""
     _check(k_pages, "k_pages")
     P, nkv, page_size, d = k_pages.shape
-    _check(v_pages, "v_pages", k_pages.dtype, _v_shape(k_pages, v_transposed))
+    _check(v_pages, "v_pages", k_pages.dtype, (P, nkv, None, None))
+    dv = v_pages.shape[2] if v_transposed else v_pages.shape[3]
+    _check(v_pages, "v_pages", k_pages.dtype, _v_shape(k_pages, v_transposed, dv))
     _check(q, "q", k_pages.dtype, contiguous=False)
     N = q.shape[0]
     if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < num_heads * d:
         raise ValueError(f"q must be [N, >= {num_heads * d}] with unit stride along rows, got {list(q.shape)}")
-    _check(out, "out", k_pages.dtype, (N, num_heads * d))
+    _check(out, "out", k_pages.dtype, (N, num_heads * dv))
+    if sink is not None:
+        _check(sink, "sink", torch.float32, (num_heads,))
     _check(block_table, "block_table", torch.int32)
     if block_table.dim() != 2:
         raise ValueError("block_table must be [requests, pages]")
@@ -732,8 +755,8 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     _call("ms_paged_attention_generic", q.data_ptr(), q.stride(0) if N > 1 else q.shape[1], k_pages.data_ptr(),
           v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], _ptr(table_rows), _ptr(n_live_tokens),
           token_req.data_ptr(), positions.data_ptr(),
-          out.data_ptr(), num_heads * d, N, num_heads, nkv, d, page_size, P, float(scale), int(window or 0),
-          int(v_transposed), _code(q.dtype), _stream())
+          out.data_ptr(), num_heads * dv, N, num_heads, nkv, d, dv, page_size, P, float(scale), int(window or 0),
+          int(v_transposed), _ptr(sink), _code(q.dtype), _stream())
     return out
 
 
@@ -843,11 +866,16 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.
 
 
 def paged_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, num_heads: int, scale: float,
-                    window: Optional[int] = None) -> torch.Tensor:
+                    window: Optional[int] = None, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of a step's tokens (``ctx``: its StepContext) over a run's pages (``kv``: its KVView).
     bfloat16 with transposed value pages and a head size the matrix-core kernel has goes there; everything
-    else (float32, other head sizes, small pages) goes to the generic kernel."""
+    else (float32, other head sizes, values of another size than keys, small pages) goes to the generic kernel.
+    ``sink`` float [num_heads]: exp(sink[h]) joins the denominator of head h's softmax."""
     d, page_size = kv.k_pages.shape[3], kv.k_pages.shape[2]
+    dv = kv.v_pages.shape[2] if kv.v_transposed else kv.v_pages.shape[3]
+    if dv != d or sink is not None:
+        return paged_attention_generic(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.token_req, ctx.positions, out,
+                                       num_heads, scale, window, kv.v_transposed, kv.table_rows, ctx.n_live_tokens, sink)
     if q.dtype == torch.bfloat16 and not (kv.v_transposed and attention_mfma_supported(d, page_size)):
         _say_once(("attention", d, page_size),
                   f"bfloat16 attention with head size {d} and pages of {page_size} tokens runs on the vector-ALU kernel: "
@@ -875,12 +903,12 @@ def _rows2d(t: torch.Tensor, name: str, dtype=None, cols=None):
 
 
 def short_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx, out: torch.Tensor,
-               mode: int = CONV_SUM, update_state: bool = True) -> torch.Tensor:
+               mode: int = CONV_SUM, update_state: bool = True, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """A causal convolution over time on every channel of ``x`` [N, C], for the step ``ctx`` describes:
     out[n] = act(sum_j weight[:, j] * input(t - taps + 1 + j)), the last column meeting the token itself, inputs before a
     request's portion taken from ``state`` [slots, taps - 1, C] (the request's slot; zero at a request's start).
     ``mode``: CONV_SUM, CONV_ADD_INPUT (x + the sum) or CONV_SILU.  With ``update_state`` the state then becomes the
-    last taps - 1 inputs of every request of the step.  ``weight`` float [C, taps]."""
+    last taps - 1 inputs of every request of the step.  ``weight`` float [C, taps]; ``bias`` float [C] is added to the sum."""
     N, C = x.shape
     xs = _rows2d(x, "x")
     os_ = _rows2d(out, "out", x.dtype, C)
@@ -891,11 +919,13 @@ def short_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx, 
     if taps > MAX_CONV_TAPS:
         raise UnsupportedShape(f"the short convolution takes up to {MAX_CONV_TAPS} taps, got {taps}")
     _check(state, "state", x.dtype, (None, max(1, taps - 1), C))
+    if bias is not None:
+        _check(bias, "bias", torch.float32, (C,))
     R = ctx.num_requests
     _check(ctx.token_req, "token_req", torch.int32, (N,))
     _check(ctx.q_start, "q_start", torch.int32, (R + 1,))
     _check(ctx.state_slots, "state_slots", torch.int32, (R,))
-    _call("ms_short_conv", x.data_ptr(), xs, weight.data_ptr(), state.data_ptr(), ctx.token_req.data_ptr(),
+    _call("ms_short_conv", x.data_ptr(), xs, weight.data_ptr(), _ptr(bias), state.data_ptr(), ctx.token_req.data_ptr(),
           ctx.q_start.data_ptr(), ctx.state_slots.data_ptr(), _ptr(ctx.n_live_tokens), out.data_ptr(), os_, N, R, C, taps,
           mode, int(update_state), int(getattr(ctx, "max_q_len", 0) == 1), _code(x.dtype), _stream())
     return out
@@ -903,12 +933,13 @@ def short_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx, 
 
 def gated_delta(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor,
                 dt_bias: torch.Tensor, state: torch.Tensor, ctx, out: torch.Tensor, heads: int, kv_heads: int, dim: int,
-                vdim: int) -> torch.Tensor:
+                vdim: int, decay_per_channel: bool = True) -> torch.Tensor:
     """The gated delta rule over the step's portions, from and into ``state`` float [slots, heads, dim, vdim]:
     per head and token  S <- g * S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q  with q, k made unit vectors
     (q also times dim^-1/2), beta = sigmoid(b), g = exp(-exp(A_log) * softplus(a + dt_bias)).  q, k [N, kv_heads * dim],
-    v [N, heads * vdim] and b [N, heads] are row slices with one row stride for q, k, v; a float [N, heads * dim];
-    out float [N, heads * vdim]."""
+    v [N, heads * vdim] and b [N, heads] are row slices with one row stride for q, k, v; a float [N, heads * dim] with
+    dt_bias [heads * dim] (a decay per head and key channel) or a float [N, heads] with dt_bias [heads] (a decay per
+    head); out float [N, heads * vdim]."""
     N = q.shape[0]
     sq = _rows2d(q, "q", None, kv_heads * dim)
     sk = _rows2d(k, "k", q.dtype, kv_heads * dim)
@@ -916,9 +947,10 @@ def gated_delta(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tens
     if not (sq == sk == sv) and N > 1:
         raise ValueError("q, k and v must be slices of rows of one width")
     sb = _rows2d(b, "b", q.dtype, heads)
-    _check(a, "a", torch.float32, (N, heads * dim))
     _check(A_log, "A_log", torch.float32, (heads,))
-    _check(dt_bias, "dt_bias", torch.float32, (heads * dim,))
+    per_channel = bool(decay_per_channel)
+    _check(a, "a", torch.float32, (N, heads * dim if per_channel else heads))
+    _check(dt_bias, "dt_bias", torch.float32, (heads * dim if per_channel else heads,))
     _check(state, "state", torch.float32, (None, heads, dim, vdim))
     _check(out, "out", torch.float32, (N, heads * vdim))
     R = ctx.num_requests
@@ -926,22 +958,26 @@ def gated_delta(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tens
     _check(ctx.state_slots, "state_slots", torch.int32, (R,))
     if heads % kv_heads:
         raise ValueError(f"{heads} heads cannot share {kv_heads} query/key heads")
-    _call("ms_gated_delta", q.data_ptr(), k.data_ptr(), v.data_ptr(), sq, a.data_ptr(), b.data_ptr(), sb, A_log.data_ptr(),
+    _call("ms_gated_delta", q.data_ptr(), k.data_ptr(), v.data_ptr(), sq, a.data_ptr(), int(per_channel), b.data_ptr(), sb,
+          A_log.data_ptr(),
           dt_bias.data_ptr(), state.data_ptr(), ctx.q_start.data_ptr(), ctx.state_slots.data_ptr(), out.data_ptr(), R,
           heads, kv_heads, dim, vdim, int(getattr(ctx, "max_q_len", 0) == 1), _code(q.dtype), _stream())
     return out
 
 
 def gated_head_norm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, out: torch.Tensor, heads: int, vdim: int,
-                    eps: float) -> torch.Tensor:
-    """out[n, h] = o[n, h] / sqrt(mean(o[n, h]^2) + eps) * weight * sigmoid(gate[n, h]); o float [N, heads * vdim]."""
+                    eps: float, gate_act: str = "sigmoid") -> torch.Tensor:
+    """out[n, h] = o[n, h] / sqrt(mean(o[n, h]^2) + eps) * weight * act(gate[n, h]), act "sigmoid" or "silu";
+    o float [N, heads * vdim]."""
+    if gate_act not in ("sigmoid", "silu"):
+        raise ValueError(f"the read-out's gate is 'sigmoid' or 'silu', not {gate_act!r}")
     N = o.shape[0]
     _check(o, "o", torch.float32, (N, heads * vdim))
     _check(weight, "weight", torch.float32, (vdim,))
     gs = _rows2d(gate, "gate", out.dtype, heads * vdim)
     _check(out, "out", None, (N, heads * vdim))
     _call("ms_gated_head_norm", o.data_ptr(), weight.data_ptr(), gate.data_ptr(), gs, out.data_ptr(), N, heads, vdim,
-          float(eps), _code(out.dtype), _stream())
+          float(eps), int(gate_act == "silu"), _code(out.dtype), _stream())
     return out
 
 
@@ -1085,4 +1121,205 @@ def latent_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, scale: float, 
           kv.block_table.shape[1], _ptr(kv.table_rows), _ptr(ctx.n_live_tokens), ctx.token_req.data_ptr(),
           ctx.positions.data_ptr(), _ptr(sink), out.data_ptr(), ot, oh, N, H, C, R, page_size, P, float(scale),
           int(window or 0), _code(q.dtype), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ norms after a sublayer
+def rms_norm_add(y: torch.Tensor, w_post: torch.Tensor, eps_post: float, x: torch.Tensor,
+                 w_next: Optional[torch.Tensor] = None, eps_next: float = 0.0,
+                 out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x += w_post * y / sqrt(mean(y^2) + eps_post), in place on the float residual stream x [N, H]; y [N, H] (rows may be
+    slices of wider rows) is a sublayer's output.  With ``out`` [N, H] also out = w_next * x / sqrt(mean(x^2) + eps_next),
+    the norm the next sublayer reads, from the same pass."""
+    _check(x, "x", torch.float32)
+    N, H = x.shape
+    ys = _rows2d(y, "y", None, H)
+    if y.shape[0] != N:
+        raise ValueError(f"y has {y.shape[0]} rows, x {N}")
+    _check(w_post, "w_post", torch.float32, (H,))
+    ocode = 0
+    if out is not None:
+        _check(out, "out", None, (N, H))
+        _check(w_next, "w_next", torch.float32, (H,))
+        ocode = _code(out.dtype)
+    _call("ms_rms_norm_add", y.data_ptr(), ys, _code(y.dtype), w_post.data_ptr(), float(eps_post), x.data_ptr(),
+          _ptr(w_next) if out is not None else None, float(eps_next), _ptr(out), ocode, N, H, _stream())
+    return out
+
+
+def add_rows(x: torch.Tensor, kept: Optional[torch.Tensor] = None, vec: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x[n] += kept[n] + vec, in place; x and kept float [N, H], vec float [H]; either addend may be left out."""
+    _check(x, "x", torch.float32)
+    N, H = x.shape
+    if kept is not None:
+        _check(kept, "kept", torch.float32, (N, H))
+    if vec is not None:
+        _check(vec, "vec", torch.float32, (H,))
+    if kept is None and vec is None:
+        return x
+    _call("ms_add_rows", x.data_ptr(), _ptr(kept), _ptr(vec), N, H, _stream())
+    return x
+
+
+def qk_norm_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                  q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                  positions: Optional[torch.Tensor] = None, coef: float = 0.0, every: int = 1,
+                  slot_mapping: Optional[torch.Tensor] = None, k_pages: Optional[torch.Tensor] = None,
+                  v_pages: Optional[torch.Tensor] = None, v_transposed: bool = False) -> torch.Tensor:
+    """In place on ``qkv`` [N, nh d + nkv d + nkv dv]: the RMS norm of every q and k head with the weights [d] (None: no
+    norm), q of the token at position p times 1 + coef * ln(floor((p + 1) / every) + 1); then k and v go into the pages
+    ([P, nkv, page, d] and [P, nkv, page, dv], or values [P, nkv, dv, page] with ``v_transposed``) at ``slot_mapping``."""
+    width = (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim
+    stride = _rows2d(qkv, "qkv", None, width)
+    N = qkv.shape[0]
+    for w, name in ((q_weight, "q_weight"), (k_weight, "k_weight")):
+        if w is not None:
+            _check(w, name, torch.float32, (head_dim,))
+    if coef:
+        _check(positions, "positions", torch.int32, (N,))
+        if every <= 0:
+            raise ValueError("the query temperature's period must be positive")
+    page_size = 0
+    if k_pages is not None:
+        _check(k_pages, "k_pages", qkv.dtype, (None, num_kv_heads, None, head_dim))
+        page_size = k_pages.shape[2]
+        _check(v_pages, "v_pages", qkv.dtype, _v_shape(k_pages, v_transposed, value_dim))
+        _check(slot_mapping, "slot_mapping", torch.int32, (N,))
+    _call("ms_qk_norm_store", qkv.data_ptr(), stride, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(positions), float(coef),
+          int(every), _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), N, num_heads, num_kv_heads, head_dim, value_dim,
+          page_size, int(bool(v_transposed)), _code(qkv.dtype), _stream())
+    return qkv
+
+
+# ------------------------------------------------------------------------------------------------ selective scan
+SCAN_MAX_STATES = 256
+
+
+def selective_scan(x: torch.Tensor, dt_in: torch.Tensor, dt_bias: torch.Tensor, A: torch.Tensor, B: torch.Tensor,
+                   C: torch.Tensor, D: torch.Tensor, z: torch.Tensor, state: torch.Tensor, ctx, out: torch.Tensor) -> torch.Tensor:
+    """The selective scan over the step's portions, from and into ``state`` float [slots, I, S]: per channel c and state n
+    S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n;  y_c = sum_n S[c, n] C_n + D_c x_c;  out = y * silu(z), with
+    dt = softplus(dt_in + dt_bias).  x, z [N, I] and B, C [N, S] are row slices (B and C of one row stride); dt_in float
+    [N, I]; A float [I, S]; D, dt_bias float [I]; out [N, I]."""
+    N, I = x.shape
+    xs = _rows2d(x, "x")
+    zs = _rows2d(z, "z", x.dtype, I)
+    S = A.shape[1]
+    bs = _rows2d(B, "B", x.dtype, S)
+    cs = _rows2d(C, "C", x.dtype, S)
+    if bs != cs and N > 1:
+        raise ValueError("B and C must be slices of rows of one width")
+    os_ = _rows2d(out, "out", x.dtype, I)
+    if z.shape[0] != N or B.shape[0] != N or C.shape[0] != N or out.shape[0] != N:
+        raise ValueError("x, z, B, C and out have one row per token")
+    _check(dt_in, "dt_in", torch.float32, (N, I))
+    _check(dt_bias, "dt_bias", torch.float32, (I,))
+    _check(A, "A", torch.float32, (I, S))
+    _check(D, "D", torch.float32, (I,))
+    _check(state, "state", torch.float32, (None, I, S))
+    R = ctx.num_requests
+    _check(ctx.q_start, "q_start", torch.int32, (R + 1,))
+    _check(ctx.state_slots, "state_slots", torch.int32, (R,))
+    _call("ms_selective_scan", x.data_ptr(), xs, dt_in.data_ptr(), dt_bias.data_ptr(), A.data_ptr(), B.data_ptr(), C.data_ptr(),
+          bs, D.data_ptr(), z.data_ptr(), zs, state.data_ptr(), ctx.q_start.data_ptr(), ctx.state_slots.data_ptr(),
+          out.data_ptr(), os_, R, I, S, _code(x.dtype), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ routed experts
+ROUTE_MAX_OUTPUTS, ROUTE_MAX_TOP = 1024, 32
+
+
+def gelu(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = x/2 (1 + erf(x / sqrt 2)), the exact gelu, worked out in float."""
+    _check(x, "x")
+    _check(out, "out", x.dtype, tuple(x.shape))
+    _call("ms_gelu", x.data_ptr(), out.data_ptr(), x.numel(), _code(x.dtype), _stream())
+    return out
+
+
+def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, n_out: Optional[int] = None):
+    """Scores = softmax(logits[:, :n_out]); the ``top`` largest of scores + correction are chosen (the lower index on a
+    tie).  Returns (ids int32 [N, top], their scores float [N, top]).  logits float [N, >= n_out]."""
+    ld = _rows2d(logits, "logits", torch.float32)
+    N = logits.shape[0]
+    n_out = logits.shape[1] if n_out is None else n_out
+    if not 0 < top <= n_out <= logits.shape[1]:
+        raise ValueError(f"top {top} of {n_out} outputs in rows of {logits.shape[1]}")
+    if correction is not None:
+        _check(correction, "correction", torch.float32, (n_out,))
+    ids = torch.empty((N, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((N, top), dtype=torch.float32, device=logits.device)
+    _call("ms_moe_route", logits.data_ptr(), ld, _ptr(correction), N, n_out, top, ids.data_ptr(), weights.data_ptr(), _stream())
+    return ids, weights
+
+
+def moe_tile_rows() -> int:
+    return int(_get("ms_moe_tile_rows")())
+
+
+def moe_align(ids: torch.Tensor, n_experts: int):
+    """Groups the rows (token, choice) of ``ids`` [N, top] by expert into tiles of ``moe_tile_rows()`` rows of one expert
+    each.  Returns (rows int32 [tiles * tile]: the flat index n * top + j of every row or -1, tile_expert int32 [tiles]:
+    the tile's expert or -1).  Choices >= n_experts (experts without weights) take no row.  The number of tiles depends
+    on the sizes alone."""
+    _check(ids, "ids", torch.int32)
+    n_items = ids.numel()
+    tile = moe_tile_rows()
+    tiles = (n_items + n_experts * (tile - 1) + tile - 1) // tile
+    rows = torch.empty(tiles * tile, dtype=torch.int32, device=ids.device)
+    tile_expert = torch.empty(tiles, dtype=torch.int32, device=ids.device)
+    _call("ms_moe_align", ids.data_ptr(), n_items, n_experts, tiles, rows.data_ptr(), tile_expert.data_ptr(), _stream())
+    return rows, tile_expert
+
+
+def grouped_gemm(a: torch.Tensor, w: torch.Tensor, rows: torch.Tensor, tile_expert: torch.Tensor, out: torch.Tensor,
+                 gather_div: int = 0, scatter: bool = False, act: Optional[str] = None) -> torch.Tensor:
+    """For every tile with an expert e and every row of it (flat position p, item = rows[p] >= 0):
+    out[item if scatter else p] = act(a[item // gather_div if gather_div else p] @ w[e].T); w [experts, n_out, K]; float
+    accumulation in the order of K.  ``act``: None or "gelu"."""
+    _check(w, "w", a.dtype)
+    if w.dim() != 3:
+        raise ValueError("w must be [experts, out features, in features]")
+    E, n_out, K = w.shape
+    a_stride = _rows2d(a, "a", None, K)
+    o_stride = _rows2d(out, "out", None, n_out)
+    tile = moe_tile_rows()
+    tiles = tile_expert.numel()
+    _check(rows, "rows", torch.int32, (tiles * tile,))
+    _check(tile_expert, "tile_expert", torch.int32)
+    if not gather_div and a.shape[0] < tiles * tile:
+        raise ValueError("a must hold a row for every row of every tile")
+    if not scatter and out.shape[0] < tiles * tile:
+        raise ValueError("out must hold a row for every row of every tile")
+    if act not in (None, "gelu"):
+        raise ValueError(f"no activation {act!r} here")
+    _call("ms_grouped_gemm", a.data_ptr(), a_stride, w.data_ptr(), rows.data_ptr(), tile_expert.data_ptr(), out.data_ptr(),
+          o_stride, tiles, n_out, K, int(gather_div), int(scatter), int(act == "gelu"), _code(a.dtype), _code(out.dtype),
+          _stream())
+    return out
+
+
+def moe_combine(part: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, h: torch.Tensor, n_experts: int,
+                out: torch.Tensor, shared: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[n] = sum_j weights[n, j] * (part[n * top + j] if ids[n, j] < n_experts else h[n]) + sigmoid(gate[n]) * shared[n].
+    part float [N * top, H]; h [N, H]; shared [N, H] (h's type or float) with gate float [N] (a column of a wider matrix
+    is fine); out float [N, H]."""
+    N, top = ids.shape
+    _check(ids, "ids", torch.int32)
+    _check(weights, "weights", torch.float32, (N, top))
+    H = out.shape[1]
+    _check(part, "part", torch.float32, (N * top, H))
+    hs = _rows2d(h, "h", None, H)
+    _check(out, "out", torch.float32, (N, H))
+    gs, scode = 0, 0
+    if shared is not None:
+        _check(shared, "shared", None, (N, H))
+        scode = _code(shared.dtype)
+        _check(gate, "gate", torch.float32, contiguous=False)
+        if gate.dim() != 1 or gate.shape[0] != N:
+            raise ValueError("gate must be one float per token")
+        gs = gate.stride(0) if N > 1 else 1
+    _call("ms_moe_combine", part.data_ptr(), ids.data_ptr(), weights.data_ptr(), h.data_ptr(), hs, _ptr(shared), scode,
+          _ptr(gate), gs, out.data_ptr(), N, top, n_experts, H, _code(h.dtype), _stream())
     return out

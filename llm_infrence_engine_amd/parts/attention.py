@@ -3,7 +3,10 @@
 q, k, v projections (one packed matrix product), position encoding fused with the cache store, causal
 attention read in place from the pages, output projection.  Query head h uses key/value head
 h // (num_heads // num_kv_heads) (src/miniserve/model.py:137-139).  Scores, softmax and the weighted
-sum are float.  ``window`` limits a query to the last ``window`` keys (None: all).
+sum are float.  ``window`` limits a query to the last ``window`` keys (None: all).  ``value_dim``: values of another
+size than queries and keys.  ``sink``: a learned number per query head (tensor ``sink`` [heads]) whose exponential joins
+the softmax's denominator; it has no key and no value and is not scaled.  ``names``: the tensors' names after the prefix,
+{"q", "k", "v", "o", "sink"} -> name; biases are the weight's name with ".bias" for ".weight".
 """
 from __future__ import annotations
 
@@ -13,35 +16,52 @@ import torch
 
 from ..kernels import linear, ops
 from ..weights.spec import TensorSpec
-from .base import KVNeed, Mixer, register_part
+from .base import CacheNeed, KVNeed, Mixer, PageTensor, register_part
+
+_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "sink": "sink"}
 
 
 class GQAttention(Mixer):
     accepts_lazy_norm = True
 
     def __init__(self, prefix: str, position, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
-                 scale: float, qkv_bias: bool = True, out_bias: bool = False, window: Optional[int] = None):
+                 scale: float, qkv_bias: bool = True, out_bias: bool = False, window: Optional[int] = None,
+                 value_dim: Optional[int] = None, sink: bool = False, names=None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads cannot share {num_kv_heads} key/value heads")
-        if head_dim % 16 or head_dim > 256:
-            raise ValueError(f"head_dim {head_dim} is not supported: the attention kernels take multiples of 16 up to 256")
+        if head_dim % 4 or head_dim > 256:
+            raise ValueError(f"head_dim {head_dim} is not supported: the attention kernels take multiples of 4 up to 256")
         if window is not None and window <= 0:
             raise ValueError("window must be positive")
         self.prefix, self.position = prefix, position
         self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
         self.scale, self.qkv_bias, self.out_bias, self.window = float(scale), qkv_bias, out_bias, window
+        self.value_dim = head_dim if value_dim is None else int(value_dim)
+        if not 0 < self.value_dim <= 256:
+            raise ValueError(f"value size {self.value_dim} is not supported: the attention kernels take up to 256")
+        if self.value_dim != head_dim and not getattr(position, "takes_value_dim", False):
+            raise ValueError("values of another size than keys need a position encoding that stores them "
+                             "(one with takes_value_dim)")
+        self.sink = bool(sink)
+        self.names = dict(_NAMES, **dict(names or {}))
+
+    def _bias_name(self, which: str) -> str:
+        name = self.names[which]
+        return name[:-len(".weight")] + ".bias" if name.endswith(".weight") else name + ".bias"
 
     # ---- weights
     def tensor_specs(self):
-        p, H, d = self.prefix, self.hidden_size, self.head_dim
+        p, H, d, dv = self.prefix, self.hidden_size, self.head_dim, self.value_dim
         specs = []
-        for name, heads in (("q_proj", self.num_heads), ("k_proj", self.num_kv_heads), ("v_proj", self.num_kv_heads)):
-            specs.append(TensorSpec(f"{p}{name}.weight", (heads * d, H)))
+        for which, rows in (("q", self.num_heads * d), ("k", self.num_kv_heads * d), ("v", self.num_kv_heads * dv)):
+            specs.append(TensorSpec(p + self.names[which], (rows, H)))
             if self.qkv_bias:
-                specs.append(TensorSpec(f"{p}{name}.bias", (heads * d,), "bias"))
-        specs.append(TensorSpec(f"{p}o_proj.weight", (H, self.num_heads * d)))
+                specs.append(TensorSpec(p + self._bias_name(which), (rows,), "bias"))
+        specs.append(TensorSpec(p + self.names["o"], (H, self.num_heads * dv)))
         if self.out_bias:
-            specs.append(TensorSpec(f"{p}o_proj.bias", (H,), "bias"))
+            specs.append(TensorSpec(p + self._bias_name("o"), (H,), "bias"))
+        if self.sink:
+            specs.append(TensorSpec(p + self.names["sink"], (self.num_heads,), "bias"))
         if self.position is not None:
             specs += self.position.tensor_specs()
         return specs
@@ -50,12 +70,13 @@ class GQAttention(Mixer):
         self.rt = rt
         by_name = {s.name: s for s in GQAttention.tensor_specs(self)}
         p = self.prefix
-        w = [get(by_name[f"{p}{n}.weight"]) for n in ("q_proj", "k_proj", "v_proj")]
+        w = [get(by_name[p + self.names[n]]) for n in ("q", "k", "v")]
         self.w_qkv = linear.prepare_weight(torch.cat(w, dim=0))
-        self.b_qkv = torch.cat([get(by_name[f"{p}{n}.bias"]) for n in ("q_proj", "k_proj", "v_proj")]).contiguous() \
+        self.b_qkv = torch.cat([get(by_name[p + self._bias_name(n)]) for n in ("q", "k", "v")]).contiguous() \
             if self.qkv_bias else None
-        self.w_o = linear.prepare_weight(get(by_name[f"{p}o_proj.weight"]))
-        self.b_o = get(by_name[f"{p}o_proj.bias"]) if self.out_bias else None
+        self.w_o = linear.prepare_weight(get(by_name[p + self.names["o"]]))
+        self.b_o = get(by_name[p + self._bias_name("o")]) if self.out_bias else None
+        self.sink_w = get(by_name[p + self.names["sink"]]) if self.sink else None
         if self.position is not None:
             self.position.load(get, rt)
 
@@ -63,8 +84,11 @@ class GQAttention(Mixer):
     def cache_need(self):
         # in bfloat16 the matrix-core attention reads value pages as an operand as they lie, transposed, which it
         # can for pages of a multiple of 16 tokens
-        return KVNeed(self.num_kv_heads, self.head_dim, self.window, transpose_values_at=16,
-                      transpose_values_in=torch.bfloat16)
+        if self.value_dim == self.head_dim:
+            return KVNeed(self.num_kv_heads, self.head_dim, self.window, transpose_values_at=16,
+                          transpose_values_in=torch.bfloat16)
+        return CacheNeed((PageTensor("k", self.num_kv_heads, self.head_dim),
+                          PageTensor("v", self.num_kv_heads, self.value_dim)), self.window)
 
     # ---- step
     def forward(self, h, ctx, kv, state):
@@ -73,9 +97,9 @@ class GQAttention(Mixer):
     def forward_residual(self, h, ctx, kv, state, x):
         if kv is None:
             raise RuntimeError("attention needs a key/value cache view")
-        nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
+        nh, nkv, d, dv = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
         q = None
-        if self.position is not None:
+        if self.position is not None and dv == d:
             q = self.position.project_encode_store(h, self.w_qkv, self.b_qkv, nh, nkv, d, ctx, kv)
         if q is None:
             # [N, (nh + 2 nkv) d]: attention reads its q part.  A library product has no bias epilogue; a position
@@ -85,12 +109,14 @@ class GQAttention(Mixer):
             q = linear.linear(h, self.w_qkv, bias=None if late_bias else self.b_qkv)
             if late_bias:
                 self.position.encode_and_store(q, nh, nkv, d, ctx, kv, bias=self.b_qkv)
+            elif dv != d:
+                self.position.encode_and_store(q, nh, nkv, d, ctx, kv, value_dim=dv)
             elif self.position is not None:
                 self.position.encode_and_store(q, nh, nkv, d, ctx, kv)
             elif kv.store:
                 ops.rope_store(q, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)
-        out = self.rt.empty(ctx.num_tokens, nh * d)
-        ops.paged_attention(q, kv, ctx, out, nh, self.scale, self.window)
+        out = self.rt.empty(ctx.num_tokens, nh * dv)
+        ops.paged_attention(q, kv, ctx, out, nh, self.scale, self.window, self.sink_w)
         return linear.linear_residual(out, self.w_o, self.b_o, x)
 
 

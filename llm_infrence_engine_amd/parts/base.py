@@ -410,6 +410,16 @@ class Block(Part):
         raise NotImplementedError
 
 
+class PassEntry(Part):
+    """What happens to the residual stream right before a pass over a stretch of layers that is walked several times."""
+
+    keeps_embedding = False    # True: ``forward`` wants the residual stream as the embedding left it
+
+    def forward(self, x: torch.Tensor, kept: Optional[torch.Tensor], t: int) -> None:
+        """Change x [N, H] (float) in place before pass ``t`` (0, 1, ...); ``kept``: the embedding's output, if asked for."""
+        raise NotImplementedError
+
+
 class Embedding(Part):
     def forward(self, ctx: StepContext) -> torch.Tensor:
         """The float residual stream [N, H] of the step's tokens."""
@@ -427,6 +437,7 @@ class Head(Part):
 # ------------------------------------------------------------------------------------------------ registries
 _REGISTRIES: Dict[str, Dict[str, type]] = {
     "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "filter": {}, "block": {}, "embedding": {}, "head": {},
+    "pass_entry": {},
 }
 
 

@@ -50,5 +50,27 @@ class ParallelResidual(Block):
         return a if b is None else b
 
 
+class SandwichResidual(Block):
+    """x <- x + post1(mixer(norm1(x)));  x <- x + post2(feed_forward(norm2(x))): every sublayer is normalised before it
+    and after it; the second norm's weight carries whatever constant the sublayer is weighted with in the sum
+    (``rms_norm(gain=...)``).  The sum into x and the norm that the next sublayer of the layer reads are one pass.
+    Without a feed-forward the layer is its first line."""
+
+    takes = {"position": "position", "mixer_norm": "norm", "mixer": "mixer", "mixer_post_norm": "norm",
+             "feed_forward_norm": "norm", "feed_forward": "feed_forward", "feed_forward_post_norm": "norm"}
+    optional = ("position", "feed_forward_norm", "feed_forward", "feed_forward_post_norm")
+
+    def forward(self, x, pending, ctx, kv, state):
+        h = self.mixer_norm.forward(x, delta=pending)
+        y = self.mixer.forward(h, ctx, kv, state)
+        if self.feed_forward is None:
+            self.mixer_post_norm.add_normed(x, y)
+            return None
+        h = self.mixer_post_norm.add_normed(x, y, then=self.feed_forward_norm)
+        self.feed_forward_post_norm.add_normed(x, self.feed_forward.forward(h, ctx))
+        return None
+
+
 register_part("block", "pre_norm_residual", PreNormResidual)
+register_part("block", "sandwich_residual", SandwichResidual)
 register_part("block", "parallel_residual", ParallelResidual)

@@ -7,12 +7,14 @@ import torch
 
 from ..kernels import linear, ops
 from ..weights.spec import TensorSpec
-from .base import Embedding, Head, register_part
+from .base import Embedding, Head, PassEntry, register_part
 
 
 class TokenEmbedding(Embedding):
-    def __init__(self, prefix: str, vocab_size: int, hidden_size: int, name: str = "weight"):
+    def __init__(self, prefix: str, vocab_size: int, hidden_size: int, name: str = "weight", scale: float = 1.0):
+        """``scale``: every row is multiplied by it on its way into the float residual stream."""
         self.prefix, self.vocab_size, self.hidden_size, self.name = prefix, vocab_size, hidden_size, name
+        self.scale = float(scale)
 
     def tensor_specs(self):
         return [TensorSpec(self.prefix + self.name, (self.vocab_size, self.hidden_size))]
@@ -23,7 +25,7 @@ class TokenEmbedding(Embedding):
 
     def forward(self, ctx):
         out = self.rt.empty(ctx.num_tokens, self.hidden_size, dtype=torch.float32)
-        return ops.embed(ctx.token_ids, self.weight, out)
+        return ops.embed(ctx.token_ids, self.weight, out, self.scale)
 
 
 class LMHead(Head):
@@ -48,5 +50,29 @@ class LMHead(Head):
         return linear.linear(h, self.weight, out_dtype=torch.float32)
 
 
+class PassStep(PassEntry):
+    """Before pass t: x <- x + e (for t > 0, with ``readd_embedding``; e is x as the embedding left it) + step[t], where
+    ``step`` is a stored table [times, hidden_size] (tensor ``name``) with one row per pass."""
+
+    def __init__(self, prefix: str, hidden_size: int, times: int, name: str = "step", readd_embedding: bool = True):
+        if times <= 0:
+            raise ValueError("a stretch of layers is walked at least once")
+        self.prefix, self.hidden_size, self.times, self.name = prefix, hidden_size, times, name
+        self.keeps_embedding = bool(readd_embedding) and times > 1
+
+    def tensor_specs(self):
+        return [TensorSpec(self.prefix + self.name, (self.times, self.hidden_size), "bias")]
+
+    def load(self, get, rt):
+        self.rt = rt
+        self.step = get(self.tensor_specs()[0])
+
+    def forward(self, x, kept, t):
+        if not 0 <= t < self.times:
+            raise ValueError(f"pass {t} of {self.times}")
+        ops.add_rows(x, kept if (t > 0 and self.keeps_embedding) else None, self.step[t])
+
+
+register_part("pass_entry", "pass_step", PassStep)
 register_part("embedding", "token_embedding", TokenEmbedding)
 register_part("head", "lm_head", LMHead)

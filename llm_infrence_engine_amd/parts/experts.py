@@ -1,0 +1,75 @@
+"""A feed-forward made of routed experts.
+
+Router logits z = W_router h in float; scores s = softmax(z) over all the router's outputs; the ``top`` outputs with the
+largest s + correction are chosen (``correction``: a stored vector that steers the choice and nothing else) and weigh in
+with their s as it is.  The first ``experts`` outputs are small feed-forwards down(act(up(h))) without biases; the last
+``identity`` outputs are experts without tensors whose output is h itself.  ``shared_ff``: one more expert of that size
+that every token runs, weighted by sigmoid(W_sg h), one number per token.
+
+Nothing here waits for the device: the tokens' choices are grouped by expert into tiles on the device, and the experts'
+products run tile by tile over a launch whose size depends on the sizes alone, so a step can be captured."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import linear, ops
+from ..weights.spec import TensorSpec
+from .base import FeedForward, register_part
+
+
+class RoutedExperts(FeedForward):
+    def __init__(self, prefix: str, hidden_size: int, expert_ff: int, experts: int, top: int, identity: int = 0,
+                 shared_ff: int = 0, activation: str = "gelu"):
+        if activation != "gelu":
+            raise ValueError(f"no activation {activation!r} for routed experts; there is 'gelu'")
+        if experts <= 0 or identity < 0 or not 0 < top <= experts + identity:
+            raise ValueError(f"{top} of {experts} + {identity} experts cannot be chosen")
+        if experts + identity > ops.ROUTE_MAX_OUTPUTS or top > ops.ROUTE_MAX_TOP:
+            raise ValueError(f"the router kernel takes up to {ops.ROUTE_MAX_OUTPUTS} outputs and a top of {ops.ROUTE_MAX_TOP}")
+        self.prefix, self.hidden_size, self.expert_ff = prefix, hidden_size, expert_ff
+        self.experts, self.identity, self.top, self.shared_ff = experts, identity, top, shared_ff
+        self.activation = activation
+
+    def tensor_specs(self):
+        p, W, F = self.prefix, self.hidden_size, self.expert_ff
+        specs = []
+        for e in range(self.experts):
+            specs += [TensorSpec(f"{p}e{e}.up", (F, W)), TensorSpec(f"{p}e{e}.down", (W, F))]
+        n_out = self.experts + self.identity
+        specs += [TensorSpec(p + "router", (n_out, W)), TensorSpec(p + "correction", (n_out,), "bias")]
+        if self.shared_ff:
+            specs += [TensorSpec(p + "shared.up", (self.shared_ff, W)), TensorSpec(p + "shared.down", (W, self.shared_ff)),
+                      TensorSpec(p + "shared.sg", (1, W))]
+        return specs
+
+    def load(self, get, rt):
+        self.rt = rt
+        t = {s.name[len(self.prefix):]: get(s) for s in self.tensor_specs()}
+        self.w_up = torch.stack([t[f"e{e}.up"] for e in range(self.experts)]).contiguous()       # [E, F, W]
+        self.w_down = torch.stack([t[f"e{e}.down"] for e in range(self.experts)]).contiguous()   # [E, W, F]
+        # the router and the shared expert's gate read the same h: one product, float out
+        self.w_router = torch.cat([t["router"]] + ([t["shared.sg"]] if self.shared_ff else []), dim=0).contiguous()
+        self.correction = t["correction"]
+        if self.shared_ff:
+            self.w_shared_up, self.w_shared_down = linear.prepare_weight(t["shared.up"]), linear.prepare_weight(t["shared.down"])
+
+    def forward(self, h, ctx):
+        N, W, E = h.shape[0], self.hidden_size, self.experts
+        n_out = E + self.identity
+        logits = ops.gemm_generic(h, self.w_router, torch.empty((N, self.w_router.shape[0]), dtype=torch.float32, device=h.device))
+        ids, weights = ops.moe_route(logits, self.correction, self.top, n_out)
+        rows, tile_expert = ops.moe_align(ids, E)
+        mid = ops.grouped_gemm(h, self.w_up, rows, tile_expert, self.rt.empty(rows.numel(), self.expert_ff),
+                               gather_div=self.top, act=self.activation)
+        part = ops.grouped_gemm(mid, self.w_down, rows, tile_expert,
+                                torch.empty((N * self.top, W), dtype=torch.float32, device=h.device), scatter=True)
+        shared = gate = None
+        if self.shared_ff:
+            u = linear.linear(h, self.w_shared_up)
+            shared = linear.linear(ops.gelu(u, torch.empty_like(u)), self.w_shared_down)
+            gate = logits[:, n_out]
+        out = torch.empty((N, W), dtype=torch.float32, device=h.device)
+        return ops.moe_combine(part, ids, weights, h, E, out, shared, gate)
+
+
+register_part("feed_forward", "routed_experts", RoutedExperts)

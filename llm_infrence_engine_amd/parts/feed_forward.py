@@ -36,9 +36,10 @@ class SwiGLU(FeedForward):
 
 class DenseAct(FeedForward):
     """down(act(up(x))), no biases.  ``activation``: "xielu", with two learned numbers (p, q) in the tensor ``act``:
-    z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2."""
+    z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2; or "gelu", the exact one,
+    z/2 (1 + erf(z / sqrt 2)), which has no tensor."""
 
-    ACTIVATIONS = ("xielu",)
+    ACTIVATIONS = ("xielu", "gelu")
 
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "xielu"):
         if activation not in self.ACTIVATIONS:
@@ -47,19 +48,21 @@ class DenseAct(FeedForward):
 
     def tensor_specs(self):
         p, H, I = self.prefix, self.hidden_size, self.intermediate_size
-        return [TensorSpec(p + "up", (I, H)), TensorSpec(p + "down", (H, I)), TensorSpec(p + "act", (2,), "bias")]
+        specs = [TensorSpec(p + "up", (I, H)), TensorSpec(p + "down", (H, I))]
+        return specs + ([TensorSpec(p + "act", (2,), "bias")] if self.activation == "xielu" else [])
 
     def load(self, get, rt):
         self.rt = rt
-        up, down, act = (get(s) for s in self.tensor_specs())
-        self.w_up, self.w_down, self.act = linear.prepare_weight(up), linear.prepare_weight(down), act
+        up, down, *act = (get(s) for s in self.tensor_specs())
+        self.w_up, self.w_down, self.act = linear.prepare_weight(up), linear.prepare_weight(down), (act[0] if act else None)
 
     def forward(self, h, ctx):
         return self.forward_residual(h, ctx, None)
 
     def forward_residual(self, h, ctx, x):
         u = linear.linear(h, self.w_up)
-        return linear.linear_residual(ops.xielu(u, self.act, torch.empty_like(u)), self.w_down, None, x)
+        u = ops.xielu(u, self.act, torch.empty_like(u)) if self.activation == "xielu" else ops.gelu(u, torch.empty_like(u))
+        return linear.linear_residual(u, self.w_down, None, x)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

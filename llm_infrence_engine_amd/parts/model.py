@@ -13,7 +13,7 @@ import torch
 from ..config.spec import ModelSpec
 from ..weights.reader import CheckpointReader, place
 from ..weights.spec import TensorSpec
-from . import attention, blocks, delta, ends, feed_forward, filters, latent, norms, positions  # noqa: F401  (register the built-in parts)
+from . import attention, blocks, delta, ends, experts, feed_forward, filters, latent, norms, positions, scan  # noqa: F401  (register the built-in parts)
 from .base import KVView, Runtime, StateView, StepContext, build_part, part_class, weakest
 
 
@@ -34,11 +34,13 @@ class Model:
             self.layers.append(part_class("block", ls.block).build(ls.parts))
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)
+        self.pass_entry = build_part("pass_entry", spec.pass_entry) if spec.pass_entry is not None else None
         self.rt: Optional[Runtime] = None
 
     # ------------------------------------------------------------------ weights
     def _parts(self):
-        return [self.embedding, *self.layers, self.final_norm, self.head]
+        return [self.embedding, *([self.pass_entry] if self.pass_entry is not None else []), *self.layers, self.final_norm,
+                self.head]
 
     def tensor_specs(self) -> List[TensorSpec]:
         """Every tensor the model wants, each name once (a tied head names the embedding's)."""
@@ -78,7 +80,8 @@ class Model:
         """Which steps of this model may be captured into graphs: True (all), "decode" (steps of single tokens)
         or False (none); the weakest answer of its parts (see ``Part.graph_safe``)."""
         return weakest([b.graph_safe() for b in self.layers] +
-                       [p.graph_safe for p in (self.embedding, self.final_norm, self.head)])
+                       [p.graph_safe for p in (self.embedding, self.final_norm, self.head)] +
+                       ([self.pass_entry.graph_safe] if self.pass_entry is not None else []))
 
     # ------------------------------------------------------------------ one step
     def forward(self, ctx: StepContext, caches: List[RunCache]) -> torch.Tensor:
@@ -90,8 +93,16 @@ class Model:
         """Embedding and all runs of the order: the float residual stream [N, H] and the last run's addend that
         is still to be summed into it (or None)."""
         x = self.embedding.forward(ctx)
+        kept = x.clone() if self.pass_entry is not None and self.pass_entry.keeps_embedding else None
         pending = None
         for i, run in enumerate(self.spec.order):
+            if run.opens_pass is not None:
+                if pending is not None:      # the pass's addends go into the sum itself
+                    from ..kernels import ops
+
+                    ops.residual_add(x, pending)
+                    pending = None
+                self.pass_entry.forward(x, kept, run.opens_pass)
             c = caches[i]
             pending = self.layers[run.layer].forward(x, pending, ctx, c.kv, c.state)
         return x, pending

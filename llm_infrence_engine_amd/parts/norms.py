@@ -1,6 +1,7 @@
-"""RMS norm: y = (offset + weight) * x * rsqrt(mean(x^2) + eps), computed in float on the float residual stream.
-``offset`` is 0 for a scale stored as it is and 1 for one stored around zero; the sum is formed once, in float,
-when the weights are loaded.
+"""RMS norm: y = gain * (offset + weight) * x * rsqrt(mean(x^2) + eps), computed in float on the float residual stream.
+``offset`` is 0 for a scale stored as it is and 1 for one stored around zero; ``gain`` is a constant of the layer (the
+weight of a normed sublayer in the residual sum, say); both are folded into the weight once, in float, when the weights
+are loaded.  ``add_normed`` is the norm of a sublayer's *output* on its way into the residual stream.
 
 The reference computes the reduction in float, casts back and multiplies by the weight in the model's
 type (src/miniserve/model.py:69-73); here the weight is applied in float too and the result is rounded once.
@@ -15,8 +16,9 @@ from .base import Norm, register_part
 
 
 class RMSNorm(Norm):
-    def __init__(self, prefix: str, size: int, eps: float, offset: float = 0.0, name: str = "weight"):
+    def __init__(self, prefix: str, size: int, eps: float, offset: float = 0.0, name: str = "weight", gain: float = 1.0):
         self.prefix, self.size, self.eps, self.offset, self.name = prefix, size, eps, float(offset), name
+        self.gain = float(gain)
 
     def tensor_specs(self):
         # a scale stored around zero is drawn around zero by the random-weights mode too
@@ -27,12 +29,24 @@ class RMSNorm(Norm):
         self.weight = get(self.tensor_specs()[0])
         if self.offset:
             self.weight = (self.weight + self.offset).contiguous()
+        if self.gain != 1.0:
+            self.weight = (self.weight * self.gain).contiguous()
 
     def forward(self, x, delta=None, rows=None, write_back=True):
         n = x.shape[0] if rows is None else rows.numel()
         out = self.rt.empty(n, self.size)
         return ops.rms_norm(x, self.weight, self.eps, out, delta=delta, rows=rows, write_back=write_back)
 
+
+    def add_normed(self, x, y, then: "RMSNorm" = None):
+        """x += this norm of y, in place on the float residual stream (y: a sublayer's output, any activation type or
+        float).  With ``then`` (another norm of the same width) also returns that norm of the new x, from the same
+        pass over the rows."""
+        if then is None:
+            ops.rms_norm_add(y, self.weight, self.eps, x)
+            return None
+        out = self.rt.empty(x.shape[0], self.size)
+        return ops.rms_norm_add(y, self.weight, self.eps, x, then.weight, then.eps, out)
 
     def forward_pair(self, other: "RMSNorm", x, delta=None):
         """(self's norm, ``other``'s norm) of the same rows of x (+ delta, kept in x): one pass when the two differ in

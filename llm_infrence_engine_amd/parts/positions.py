@@ -82,6 +82,46 @@ class RotaryPairs(PositionEncoding):
         return ops.rotary_pairs(src, dst, ctx.positions, self.inv_freq)
 
 
+class QKNormTemperature(PositionEncoding):
+    """Heads that are normalised instead of rotated.  Every query and key head passes an RMS norm with a weight of
+    its own kind (``q_norm`` / ``k_norm`` [head_dim], shared by the heads; ``qk_norm`` False: no norm), and the position
+    enters through a query temperature alone: q of the token at position p is multiplied by
+    1 + coef * ln(floor((p + 1) / every) + 1) (``coef`` 0 or None: no temperature).  Keys and values may differ in size.
+    Norm, logarithm and temperature are float; one kernel also stores k and v into the pages."""
+
+    takes_value_dim = True
+
+    def __init__(self, prefix: str, head_dim: int, eps: float, qk_norm: bool = True, coef: float = 0.0, every: int = 1,
+                 q_norm_name: str = "q.norm", k_norm_name: str = "k.norm"):
+        if coef and every <= 0:
+            raise ValueError("the query temperature's period must be positive")
+        self.prefix, self.head_dim, self.eps, self.qk_norm = prefix, head_dim, float(eps), bool(qk_norm)
+        self.coef, self.every = float(coef or 0.0), int(every)
+        self.q_norm_name, self.k_norm_name = q_norm_name, k_norm_name
+        self.q_weight = self.k_weight = None
+
+    def tensor_specs(self):
+        if not self.qk_norm:
+            return []
+        from ..weights.spec import TensorSpec
+
+        return [TensorSpec(self.prefix + self.q_norm_name, (self.head_dim,), "norm"),
+                TensorSpec(self.prefix + self.k_norm_name, (self.head_dim,), "norm")]
+
+    def load(self, get, rt):
+        self.rt = rt
+        if self.qk_norm:
+            self.q_weight, self.k_weight = (get(s) for s in self.tensor_specs())
+
+    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, kv, value_dim=None):
+        store = kv is not None and kv.store
+        ops.qk_norm_store(qkv, num_heads, num_kv_heads, head_dim, head_dim if value_dim is None else value_dim,
+                          self.q_weight, self.k_weight, self.eps, ctx.positions, self.coef, self.every,
+                          kv.slot_mapping if store else None, kv.k_pages if store else None,
+                          kv.v_pages if store else None, bool(store and kv.v_transposed))
+
+
+register_part("position", "qk_norm_temperature", QKNormTemperature)
 register_part("position", "rotary_half", RotaryHalf)
 register_part("position", "rotary_pairs", RotaryPairs)
 register_part("position", "none", NoPosition)
