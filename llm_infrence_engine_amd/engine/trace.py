@@ -19,7 +19,7 @@ from pathlib import Path
 
 PAGE_SIZE = 16        # tokens per page
 ROUND_TO = 64         # --max-tokens counts each live request rounded up to this many tokens
-MAX_LIVE = 8          # request rows (the format allows up to four live requests; leave room)
+MAX_LIVE = 4          # request rows: the format allows up to four live requests
 
 
 def replay(model_dir, dtype: str, out_dir, max_tokens: int, lines, log=sys.stdout, page_size: int = PAGE_SIZE,

@@ -45,6 +45,17 @@ def read_weights(model_dir, dtype=torch.float64) -> dict:
 
 
 # --------------------------------------------------------------------------- small pieces
+def same(x):
+    return x
+
+
+def rounder(act_dtype):
+    """x as an engine that stores activations in ``act_dtype`` would hold it (None: exact).  Used only to measure how far
+    a faithful reduced-precision computation strays from the exact one; ``rd`` below is such a function, applied to
+    what the products and the convolutions leave (never to the residual stream, norms, decays or states)."""
+    return same if act_dtype is None else (lambda x: x.to(act_dtype).to(x.dtype))
+
+
 def rms(x: torch.Tensor, eps: float) -> torch.Tensor:
     """x divided by its root mean square over the last dimension, eps inside the root."""
     return x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps)
@@ -109,24 +120,24 @@ def delta_recurrence(q, k, v, g, beta, S0=None):
     return o, S
 
 
-def delta_mixer(h, w, p, m, eps):
+def delta_mixer(h, w, p, m, eps, rd=same):
     """h [T, W]; w: the tensors; p: the layer's prefix ('l3.mix.'); m: the mixer's sizes."""
     T = h.shape[0]
     H, G, D, E = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = silu(causal_conv(h @ w[p + "q"].T, w[p + "q.conv"])).reshape(T, G, D)
-    k = silu(causal_conv(h @ w[p + "k"].T, w[p + "k.conv"])).reshape(T, G, D)
-    v = silu(causal_conv(h @ w[p + "v"].T, w[p + "v.conv"])).reshape(T, H, E)
+    q = rd(silu(causal_conv(rd(h @ w[p + "q"].T), w[p + "q.conv"]))).reshape(T, G, D)
+    k = rd(silu(causal_conv(rd(h @ w[p + "k"].T), w[p + "k.conv"]))).reshape(T, G, D)
+    v = rd(silu(causal_conv(rd(h @ w[p + "v"].T), w[p + "v.conv"]))).reshape(T, H, E)
     q = unit(q) * D ** -0.5
     k = unit(k)
     rep = H // G
     q = q.repeat_interleave(rep, dim=1)
     k = k.repeat_interleave(rep, dim=1)
-    beta = torch.sigmoid(h @ w[p + "b"].T)
+    beta = torch.sigmoid(rd(h @ w[p + "b"].T))
     g = delta_decay(h, w[p + "a"], w[p + "A_log"], w[p + "dt_bias"])
     o, _ = delta_recurrence(q, k, v, g, beta)
     o = rms(o, eps) * w[p + "norm"]
-    o = o * silu(h @ w[p + "g"].T).reshape(T, H, E)
-    return o.reshape(T, H * E) @ w[p + "o"].T
+    o = rd(o * silu(rd(h @ w[p + "g"].T)).reshape(T, H, E))
+    return rd(o.reshape(T, H * E) @ w[p + "o"].T)
 
 
 # --------------------------------------------------------------------------- mixer: attention
@@ -151,22 +162,23 @@ def sink_softmax_attention(q, k, v, scale, sink):
     return out
 
 
-def attention_mixer(h, w, p, m, eps):
+def attention_mixer(h, w, p, m, eps, rd=same):
     T = h.shape[0]
     H, G, D, E = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = (h @ w[p + "q"].T).reshape(T, H, D)
-    k = (h @ w[p + "k"].T).reshape(T, G, D)
-    v = (h @ w[p + "v"].T).reshape(T, G, E)
+    q = rd(h @ w[p + "q"].T).reshape(T, H, D)
+    k = rd(h @ w[p + "k"].T).reshape(T, G, D)
+    v = rd(h @ w[p + "v"].T).reshape(T, G, E)
     q = norm(q, w[p + "q.norm"], eps)
-    k = norm(k, w[p + "k.norm"], eps)
+    k = rd(norm(k, w[p + "k.norm"], eps))
     temp = m.get("q_temp")
     if temp is not None:
         q = q * query_temperature(T, temp["coef"], temp["every"], h.dtype)[:, None, None]
+    q = rd(q)
     rep = H // G
     k = k.repeat_interleave(rep, dim=1)
     v = v.repeat_interleave(rep, dim=1)
-    o = sink_softmax_attention(q, k, v, m["scale"], w[p + "sink"])
-    return o.reshape(T, H * E) @ w[p + "o"].T
+    o = rd(sink_softmax_attention(q, k, v, m["scale"], w[p + "sink"]))
+    return rd(o.reshape(T, H * E) @ w[p + "o"].T)
 
 
 # --------------------------------------------------------------------------- mixer: selective scan
@@ -182,22 +194,22 @@ def selective_scan(x, dt, A, B, C, Dskip, S0=None):
     return y, S
 
 
-def mamba_mixer(h, w, p, m):
+def mamba_mixer(h, w, p, m, rd=same):
     I, N, R = m["inner"], m["state"], m["dt_rank"]
-    xz = h @ w[p + "in"].T
+    xz = rd(h @ w[p + "in"].T)
     x, z = xz[:, :I], xz[:, I:]
-    x = silu(causal_conv(x, w[p + "conv"], w[p + "conv.b"]))
-    proj = x @ w[p + "x"].T
+    x = rd(silu(causal_conv(x, w[p + "conv"], w[p + "conv.b"])))
+    proj = rd(x @ w[p + "x"].T)
     dt, B, C = proj[:, :R], proj[:, R:R + N], proj[:, R + N:]
     dt = softplus(dt @ w[p + "dt"].T + w[p + "dt.b"])
     A = -torch.exp(w[p + "A_log"])
     y, _ = selective_scan(x, dt, A, B, C, w[p + "D"])
-    return (y * silu(z)) @ w[p + "o"].T
+    return rd(rd(y * silu(z)) @ w[p + "o"].T)
 
 
 # --------------------------------------------------------------------------- feed-forward
-def dense_ff(h, up, down):
-    return gelu_erf(h @ up.T) @ down.T
+def dense_ff(h, up, down, rd=same):
+    return rd(rd(gelu_erf(rd(h @ up.T))) @ down.T)
 
 
 def route(h, w_router, correction, top: int):
@@ -208,7 +220,7 @@ def route(h, w_router, correction, top: int):
     return chosen, torch.gather(s, 1, chosen)
 
 
-def moe_ff(h, w, p, mlp):
+def moe_ff(h, w, p, mlp, rd=same):
     r = mlp["router"]
     n_real, n_id, top = r["experts"], r.get("identity", 0), r["top"]
     chosen, weights = route(h, w[p + "router"], w[p + "correction"], top)
@@ -220,19 +232,19 @@ def moe_ff(h, w, p, mlp):
                 assert e < n_real + n_id
                 y = h[t]
             else:
-                y = dense_ff(h[t:t + 1], w[f"{p}e{e}.up"], w[f"{p}e{e}.down"])[0]
+                y = dense_ff(h[t:t + 1], w[f"{p}e{e}.up"], w[f"{p}e{e}.down"], rd)[0]
             out[t] += weights[t, j] * y
     if mlp.get("shared") is not None:
         gate = torch.sigmoid(h @ w[p + "shared.sg"].T)          # [T, 1]
-        out = out + gate * dense_ff(h, w[p + "shared.up"], w[p + "shared.down"])
+        out = out + gate * dense_ff(h, w[p + "shared.up"], w[p + "shared.down"], rd)
     return out
 
 
-def feed_forward(h, w, p, mlp):
+def feed_forward(h, w, p, mlp, rd=same):
     if mlp["kind"] == "dense":
-        return dense_ff(h, w[p + "up"], w[p + "down"])
+        return dense_ff(h, w[p + "up"], w[p + "down"], rd)
     if mlp["kind"] == "moe":
-        return moe_ff(h, w, p, mlp)
+        return moe_ff(h, w, p, mlp, rd)
     raise ValueError(mlp["kind"])
 
 
@@ -252,41 +264,43 @@ def layer_order(cfg: dict):
     return order
 
 
-def run_layer(x, i, entry, w, cfg):
-    eps, m = cfg["norm"]["eps"], cfg["residual_mult"]
+def run_layer(x, i, entry, w, cfg, rd=same):
+    eps, m = cfg["norm"]["eps"], cfg.get("residual_mult", 1.0)
     p = f"l{i}."
-    h = norm(x, w[p + "norm1"], eps)
+    h = rd(norm(x, w[p + "norm1"], eps))
     kind = entry["type"]
     if kind == "delta":
-        y = delta_mixer(h, w, p + "mix.", entry["mixer"], eps)
+        y = delta_mixer(h, w, p + "mix.", entry["mixer"], eps, rd)
     elif kind == "attention":
-        y = attention_mixer(h, w, p + "mix.", entry["mixer"], eps)
+        y = attention_mixer(h, w, p + "mix.", entry["mixer"], eps, rd)
     elif kind == "mamba1":
-        y = mamba_mixer(h, w, p + "mix.", entry["mixer"])
+        y = mamba_mixer(h, w, p + "mix.", entry["mixer"], rd)
     else:
         raise ValueError(kind)
     x = x + m * norm(y, w[p + "norm1b"], eps)
     if entry.get("mlp") is not None:
-        y = feed_forward(norm(x, w[p + "norm2"], eps), w, p + "mlp.", entry["mlp"])
+        y = feed_forward(rd(norm(x, w[p + "norm2"], eps)), w, p + "mlp.", entry["mlp"], rd)
         x = x + m * norm(y, w[p + "norm2b"], eps)
     return x
 
 
-def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out=None) -> torch.Tensor:
-    """Logits [T, vocab] of one sequence.  ``layers_out``: a list that receives x after every layer run."""
+def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out=None, act_dtype=None) -> torch.Tensor:
+    """Logits [T, vocab] of one sequence.  ``layers_out``: a list that receives x after every layer run.  ``act_dtype``:
+    round what lies between the products as an engine of that type would (see ``rounder``)."""
+    rd = rounder(act_dtype)
     w = {k: v.to(dtype) for k, v in w.items()}
     ids = torch.as_tensor(tokens, dtype=torch.long)
-    x = w["embed"][ids] * cfg["embedding"]["scale"]
+    x = w["embed"][ids] * (cfg.get("embedding") or {}).get("scale", 1.0)
     e = x.clone()
     for i, t in layer_order(cfg):
         if t is not None:
             if t > 0:
                 x = x + e
             x = x + w["loop.step"][t]
-        x = run_layer(x, i, cfg["layers"][i], w, cfg)
+        x = run_layer(x, i, cfg["layers"][i], w, cfg, rd)
         if layers_out is not None:
             layers_out.append(x.clone())
-    return norm(x, w["final.norm"], cfg["norm"]["eps"]) @ w["head"].T
+    return rd(norm(x, w["final.norm"], cfg["norm"]["eps"])) @ w["head"].T
 
 
 def greedy(cfg, w, prompt, n_new, dtype=torch.float64):
