@@ -22,7 +22,9 @@ them out.  ``--only sample`` times the sampler alone at the real vocabulary.
 ``--design gemadra`` measures another design instead: the Gemadra decoder (delta-rule and latent-attention layers in
 turn) beside the Qwen2 decoder at the same width, depth and feed-forward weights, a 2,048-token prompt in one step
 and decode steps at batch 8 and 64, at the widths of the 0.5B and the 7B shape (``--design-layers`` layers each,
-random weights, bfloat16); one JSON line, ``sizes[width][design]``.
+random weights, bfloat16); one JSON line, ``sizes[width][design]``.  ``--design gidurax`` does the same for the Gidurax
+decoder (selective scan, delta rule with a decay per head, two attention layers with a sink; every second feed-forward
+routed over sixteen experts) beside Gemadra and Qwen2.
 """
 from __future__ import annotations
 
@@ -255,22 +257,25 @@ def generic_costs(model, cfg_dict=None):
 
 
 def run_design(eng, a):
-    """Gemadra beside Qwen2 at equal width, depth and feed-forward weights."""
+    """Another design beside the closest existing ones at equal width, depth and feed-forward weights: Gemadra beside
+    Qwen2; Gidurax beside Gemadra and Qwen2."""
     import gc
 
     import torch
 
     from llm_infrence_engine_amd.config import config_from_dict, preset
 
-    out = {"design": "gemadra", "beside": "qwen2", "layers": a.design_layers, "dtype": "bf16", "data": "synthetic",
+    beside = ["qwen2"] if a.design == "gemadra" else ["gemadra", "qwen2"]
+    out = {"design": a.design, "beside": ",".join(beside), "layers": a.design_layers, "dtype": "bf16", "data": "synthetic",
            "prefill_tokens": PREFILL_TOKENS, "prompt_len": a.prompt_len, "sizes": {}}
     for size in a.design_sizes.split(","):
         row = {}
-        for design, name in (("gemadra", "gemadra-" + size), ("qwen2", size)):
+        for design in [a.design] + beside:
+            name = size if design == "qwen2" else f"{design}-{size}"
             if a.design_only not in (None, design):
                 continue
             d = preset(name)
-            if design == "gemadra":
+            if design != "qwen2":
                 d["layers"] = d["layers"][:a.design_layers]
             else:
                 d["num_hidden_layers"] = a.design_layers
@@ -300,13 +305,14 @@ def run_design(eng, a):
 
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
-    ap.add_argument("--design", choices=["gemadra"], default=None,
-                    help="measure this design beside the Qwen2 decoder at equal sizes instead of the default workload")
+    ap.add_argument("--design", choices=["gemadra", "gidurax"], default=None,
+                    help="measure this design beside the closest existing ones (Gemadra beside Qwen2; Gidurax beside "
+                         "Gemadra and Qwen2) at equal sizes instead of the default workload")
     ap.add_argument("--design-layers", type=int, default=4, help="layers of each model in a --design run")
     ap.add_argument("--design-sizes", default="0.5b,7b", help="widths of a --design run (0.5b, 7b)")
     ap.add_argument("--design-part", choices=["all", "prefill", "decode"], default="all",
                     help="a --design run's prompt step or its decode steps alone (for profiles)")
-    ap.add_argument("--design-only", choices=["gemadra", "qwen2"], default=None,
+    ap.add_argument("--design-only", choices=["gemadra", "gidurax", "qwen2"], default=None,
                     help="one of the two models of a --design run alone (for profiles)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)

@@ -1,5 +1,5 @@
 """Named config.json contents for the random-weights mode: the shapes the published Qwen2.5 checkpoints
-have, the two tiny ones the tests use and two Gemadra shapes of the same widths, so that ``--random-config 0.5b``
+have, the two tiny ones the tests use and two Gemadra and two Gidurax shapes of the same widths, so that ``--random-config 0.5b``
 needs no file.  These are data
 of the kind a config.json holds; no part or kernel reads them.
 """
@@ -43,6 +43,32 @@ PRESETS["gemadra-7b"] = _gemadra(
     {"heads": 28, "kv_heads": 14, "dim": 128, "vdim": 128, "conv": 4, "decay_rank": 128, "gate_rank": 128},
     {"heads": 28, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": 1536, "mask": {"size": 1024},
      "rot": {"base": 10000.0, "dims": 64}, "scale": 192 ** -0.5}, vocab=152064)
+
+
+def _gidurax(width, ff, layers, scan, delta, attention, experts, vocab=151936):
+    """``layers`` layers in the order scan, delta rule, attention, attention; every second one with routed experts
+    (``experts``: (expert ff, experts, identities, top, shared ff)), the others with a dense feed-forward."""
+    ef, n, ident, top, shared = experts
+    routed = {"kind": "moe", "expert": {"ff": ef}, "router": {"experts": n, "identity": ident, "top": top}, "shared": {"ff": shared}}
+    kinds = [("mamba1", scan), ("delta", delta), ("attention", attention), ("attention", attention)]
+    return {"architecture": "Gidurax", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.7,
+            "embedding": {"scale": float(width) ** 0.5},
+            "layers": [{"type": kinds[i % 4][0], "mixer": dict(kinds[i % 4][1]),
+                        "mlp": dict(routed) if i % 2 else {"kind": "dense", "ff": ff}} for i in range(layers)]}
+
+
+# Gidurax at the same widths: dense feed-forwards of Gemadra's size, routed ones whose chosen experts and shared expert
+# together have about as many weights (three of sixteen experts and two identities, plus the shared one)
+PRESETS["gidurax-0.5b"] = _gidurax(
+    896, 7296, 24, {"inner": 1792, "state": 16, "dt_rank": 56, "conv": 4},
+    {"heads": 14, "kv_heads": 7, "dim": 64, "vdim": 64, "conv": 4},
+    {"heads": 14, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.125, "q_temp": {"coef": 0.3, "every": 128}},
+    (1824, 16, 2, 3, 1824))
+PRESETS["gidurax-7b"] = _gidurax(
+    3584, 28416, 28, {"inner": 7168, "state": 16, "dt_rank": 224, "conv": 4},
+    {"heads": 28, "kv_heads": 14, "dim": 128, "vdim": 128, "conv": 4},
+    {"heads": 28, "kv_heads": 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "q_temp": {"coef": 0.3, "every": 128}},
+    (7104, 16, 2, 3, 7104), vocab=152064)
 
 
 def preset(name: str) -> dict:

@@ -115,7 +115,7 @@ int ms_paged_attention_mfma(const void* q, long long q_stride, const void* k_pag
                             const int* block_table, int table_stride, const int* table_rows, const int* q_start,
                             const int* context_lens, void* out, long long out_stride, int n_requests, int n_tokens,
                             int max_q_len, int num_heads, int num_kv_heads, int head_dim, int page_size, float scale,
-                            int window, hipStream_t stream);
+                            int window, const float* sink, hipStream_t stream);
 
 int ms_paged_attention_mfma_decode(const void* q, long long q_stride, const void* k_pages, const void* vt_pages,
                                    const int* block_table, int table_stride, const int* table_rows,
@@ -123,7 +123,7 @@ int ms_paged_attention_mfma_decode(const void* q, long long q_stride, const void
                                    void* part_o,
                                    void* part_ml, int n_requests, int num_heads, int num_kv_heads, int head_dim,
                                    int page_size, float scale, int window, int min_blocks, int n_splits,
-                                   hipStream_t stream);
+                                   const float* sink, hipStream_t stream);
 
 int ms_argmax(const float* logits, long long ld, int n_rows, int vocab, float* scratch_val, int* scratch_idx,
               int n_chunks, int* out, hipStream_t stream);
@@ -235,13 +235,16 @@ int ms_gelu(const void* x, void* out, long long total, int dtype, hipStream_t st
 int ms_moe_route(const float* logits, long long ld, const float* correction, int n_tokens, int n_out, int top, int* ids,
                  float* weights, hipStream_t stream);
 int ms_moe_tile_rows();
-// rows [tiles * ms_moe_tile_rows()] and tile_expert [tiles] from ids [n_items]; ids >= n_experts take no row
-int ms_moe_align(const int* ids, int n_items, int n_experts, int tiles, int* rows, int* tile_expert, hipStream_t stream);
+// rows [tiles * tile] and tile_expert [tiles] from ids [n_items]; ids >= n_experts take no row; tile: ms_moe_tile_rows()
+// or four times that (for the matrix-core product alone)
+int ms_moe_align(const int* ids, int n_items, int n_experts, int tile, int tiles, int* rows, int* tile_expert,
+                 hipStream_t stream);
+int ms_grouped_gemm_mfma_ok(int K, long long in_stride, long long out_stride, int tile, int dtype, int out_dtype);
 // for every tile t with an expert e and each of its rows i (flat position p = t * tile + i, item = rows[p] >= 0):
 // out[out_scatter ? item : p] = act(w[e] . in[in_div ? item / in_div : p]); w [experts, n_out, K]
 int ms_grouped_gemm(const void* in, long long in_stride, const void* w, const int* rows, const int* tile_expert, void* out,
-                    long long out_stride, int tiles, int n_out, int K, int in_div, int out_scatter, int act, int dtype,
-                    int out_dtype, hipStream_t stream);
+                    long long out_stride, int tiles, int tile, int n_out, int K, int in_div, int out_scatter, int act,
+                    int dtype, int out_dtype, hipStream_t stream);
 int ms_moe_combine(const float* part, const int* ids, const float* weights, const void* h, long long h_stride,
                    const void* shared, int shared_dtype, const float* gate, long long gate_stride, float* out,
                    int n_tokens, int top, int n_experts, int hidden, int dtype, hipStream_t stream);

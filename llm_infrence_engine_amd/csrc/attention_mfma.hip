@@ -114,14 +114,15 @@ __device__ __forceinline__ void load_values(ValueBlock<CT>& b, const bf16* __res
 // but only D / VS of the output's dims, so it reads all keys and 1 / VS of the values.  A compute unit draws
 // its data at a small fraction of the chip's rate, so when a step has fewer tiles than the chip has units this
 // shortens the longest chain without a second kernel; the blocks write disjoint dims and share nothing.
-template <int D, int NT, int WAVES, bool SPLIT, int VS>
+template <int D, int NT, int WAVES, bool SPLIT, int VS, bool SINK>
 __global__ void __launch_bounds__(WAVES * MS_WAVE, (NT > 1 ? 2 : 1))
 attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* __restrict__ k_pages,
                       const bf16* __restrict__ vt_pages, const int* __restrict__ block_table, int table_stride,
                       const int* __restrict__ table_rows, const int* __restrict__ q_start,
                       const int* __restrict__ context_lens, bf16* __restrict__ out, size_t out_stride,
                       float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int page_size,
-                      int page_shift, float scale_log2e, int window, int min_blocks, int n_splits) {
+                      int page_shift, float scale_log2e, int window, int min_blocks, int n_splits,
+                      const float* __restrict__ sink) {
   // SPLIT: min_blocks and n_splits say how a request's key blocks are spread.  Else min_blocks != 0 asks for
   // the order of tiles in which a long tile's companion on its CU is a short one (see below), and n_splits is
   // the number of requests whose tiles the grid's second dimension runs over (0: one tile to a request)
@@ -257,6 +258,18 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
     if (SUMS_BY_MATRIX) lsum[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int c = 0; c < CT; ++c) o[c][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  // A sink is one more term of the denominator with no key and no value: the running softmax of one wave (the first
+  // wave of the block, of the first split) starts as if it had already seen a key with that score, unscaled, and a
+  // value of zero.  Everything after (moving the reference, merging waves and splits) treats it as any other term.
+  if (SINK && wave == 0 && (!SPLIT || bx == 0)) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int cc = min(c0 + t * 16 + col16, ncols - 1);
+      m[t] = sink[g * rep + cc % rep] * 1.4426950408889634f;
+      lvec[t] = kq == 0 ? 1.0f : 0.f;
+      if (SUMS_BY_MATRIX) lsum[t] = f32x4{1.f, 1.f, 1.f, 1.f};
+    }
   }
 
   // A narrow tile (decode) has registers to spare and few waves to hide a wait behind: it fetches the next
@@ -538,7 +551,7 @@ template <int D, int NT, int WAVES, int VS>
 int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
                    const int* table_rows, const int* q_start, const int* ctx, bf16* out, size_t out_stride,
                    int n_requests, int n_tokens, int max_q_len, int nh, int nkv, int page_size, float scale,
-                   int window, hipStream_t stream) {
+                   int window, const float* sink, hipStream_t stream) {
   const int rep = nh / nkv;
   const long long per_request = ((long long)max_q_len * rep + 16 * NT - 1) / (16 * NT);
   // every request may end in a partial tile; no step has more tiles than if each request were the longest
@@ -548,7 +561,13 @@ int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt
   const int pair_order = tiles * VS * nkv <= 2LL * ms_compute_units() ? 1 : 0;
   const int scan = per_request == 1 ? 0 : n_requests;   // one tile to a request: the tile's index is the request's
   dim3 grid(nkv, (unsigned)tiles, VS), block(WAVES * MS_WAVE);
-  attention_mfma_kernel<D, NT, WAVES, false, VS><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, pair_order, scan);
+  if constexpr (D == 64 && NT == 4) {     // no variant with a sink at this shape (its registers are spent)
+    if (sink) return MS_UNSUPPORTED;
+  } else if (sink) {
+    attention_mfma_kernel<D, NT, WAVES, false, VS, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, pair_order, scan, sink);
+    return ms_launch_status();
+  }
+  attention_mfma_kernel<D, NT, WAVES, false, VS, false><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, pair_order, scan, nullptr);
   return ms_launch_status();
 }
 
@@ -556,9 +575,12 @@ template <int D>
 int launch_split(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
                  const int* table_rows, const int* q_start, const int* ctx, bf16* out, size_t out_stride, float* part_o, float* part_ml,
                  int n_requests, int nh, int nkv, int page_size, float scale, int window, int min_blocks,
-                 int n_splits, hipStream_t stream) {
+                 int n_splits, const float* sink, hipStream_t stream) {
   dim3 grid(n_splits, nkv, n_requests), block(4 * MS_WAVE);
-  attention_mfma_kernel<D, 1, 4, true, 1><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, min_blocks, n_splits);
+  if (sink)
+    attention_mfma_kernel<D, 1, 4, true, 1, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, min_blocks, n_splits, sink);
+  else
+    attention_mfma_kernel<D, 1, 4, true, 1, false><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, min_blocks, n_splits, nullptr);
   attention_combine_kernel<D><<<dim3(n_requests * nh), dim3(D < 64 ? 64 : D), 0, stream>>>(part_o, part_ml, q_start, ctx, out, out_stride, nh, window, min_blocks, n_splits);
   return ms_launch_status();
 }
@@ -589,14 +611,15 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
                                        const int* block_table, int table_stride, const int* table_rows,
                                        const int* q_start, const int* context_lens, void* out, long long out_stride,
                                        int n_requests, int n_tokens, int max_q_len, int num_heads, int num_kv_heads,
-                                       int head_dim, int page_size, float scale, int window, hipStream_t stream) {
+                                       int head_dim, int page_size, float scale, int window, const float* sink,
+                                       hipStream_t stream) {
   if (n_requests <= 0 || max_q_len <= 0 || n_tokens <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || table_stride <= 0) return MS_BAD_ARG;
   if (!(scale > 0.f)) return MS_BAD_ARG;   // maxima are taken of the raw scores
   if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
-#define GO(D, NT, WV, VS) return launch_general<D, NT, WV, VS>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, table_rows, q_start, context_lens, (bf16*)out, out_stride, n_requests, n_tokens, max_q_len, num_heads, num_kv_heads, page_size, scale, window, stream)
+#define GO(D, NT, WV, VS) return launch_general<D, NT, WV, VS>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, table_rows, q_start, context_lens, (bf16*)out, out_stride, n_requests, n_tokens, max_q_len, num_heads, num_kv_heads, page_size, scale, window, sink, stream)
   // Tile width (NT * 16 columns) and waves over a tile's keys.  Few columns (a decode step): one narrow tile
   // per request and many waves over its keys.
   const int cols = max_q_len * (num_heads / num_kv_heads);
@@ -615,6 +638,8 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
     while (vs < 4 && (head_dim / 16) % (vs * 2) == 0 && tiles * vs * 2 <= cus) vs *= 2;
     if (head_dim == 128 && tiles >= 2LL * cus) waves = 4;
   }
+  // with a sink the widest tile at head size 64 has no register left for the softmax's other starting point
+  if (sink != nullptr && head_dim == 64 && nt == 4) nt = 2;
   if (g_force_nt) { nt = g_force_nt; waves = g_force_waves; }
   if (g_force_vs) vs = g_force_vs;
   if (nt > 1) vs = 1;
@@ -642,7 +667,7 @@ extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride,
                                               const int* table_rows, const int* q_start, const int* context_lens, void* out,
                                               long long out_stride, void* part_o, void* part_ml, int n_requests,
                                               int num_heads, int num_kv_heads, int head_dim, int page_size,
-                                              float scale, int window, int min_blocks, int n_splits,
+                                              float scale, int window, int min_blocks, int n_splits, const float* sink,
                                               hipStream_t stream) {
   if (n_requests <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || table_stride <= 0) return MS_BAD_ARG;
@@ -652,7 +677,7 @@ extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride,
   if (min_blocks <= 0 || n_splits <= 0 || n_splits > COMBINE_MAX_SPLITS) return MS_BAD_ARG;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)part_o % 16)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
-#define GO(D) return launch_split<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, table_rows, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, min_blocks, n_splits, stream)
+#define GO(D) return launch_split<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, table_rows, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, min_blocks, n_splits, sink, stream)
   if (head_dim == 32) GO(32);
   if (head_dim == 64) GO(64);
   GO(128);

@@ -167,6 +167,84 @@ grouped_gemm_kernel(const T* __restrict__ in, size_t in_stride, const T* __restr
   }
 }
 
+// The same product on the matrix cores, bfloat16 in, K a multiple of 32.  A block owns one tile of 16 * NT rows and a slab
+// of 128 output features, 32 to each of its four waves: the expert's rows are the A operand of
+// v_mfma_f32_16x16x32_bf16 (a lane reads 16 bytes of a row), the tile's activations, gathered by the rows' list, the B
+// operand; a lane then holds four neighbouring features of one row.  Every output sums over k in the same order whatever
+// else is in the tile.  The grid runs over slabs first, so that neighbouring blocks read the same activations and
+// different weights.
+typedef __attribute__((ext_vector_type(8))) __bf16 gg_bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 gg_bf16x4;
+typedef __attribute__((ext_vector_type(4))) float gg_f32x4;
+constexpr int GG_SLAB = 128;
+
+template <int NT, typename TO>
+__global__ void __launch_bounds__(256)
+grouped_gemm_mfma_kernel(const bf16* __restrict__ in, size_t in_stride, const bf16* __restrict__ w,
+                         const int* __restrict__ rows, const int* __restrict__ tile_expert, TO* __restrict__ out,
+                         size_t out_stride, int n_out, int K, int in_div, int out_scatter, int act) {
+  constexpr int TM = 16 * NT;
+  const int tile = blockIdx.y;
+  const int e = tile_expert[tile];
+  if (e < 0) return;
+  const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
+  const int col = lane & 15, kq = lane >> 4;
+  const int f0 = blockIdx.x * GG_SLAB + wave * 32;
+  if (f0 >= n_out) return;
+  const bf16* we = w + (size_t)e * n_out * K;
+  const bf16* wrow[2];
+  bool wlive[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int f = f0 + u * 16 + col;
+    wlive[u] = f < n_out;
+    wrow[u] = we + (size_t)(wlive[u] ? f : 0) * K + kq * 8;
+  }
+  const bf16* arow[NT];
+  int item[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int p = tile * TM + t * 16 + col;
+    item[t] = rows[p];
+    const size_t src = in_div > 0 ? (size_t)(max(item[t], 0) / in_div) : (size_t)p;
+    arow[t] = in + src * in_stride + kq * 8;
+  }
+  gg_f32x4 acc[2][NT];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[u][t] = gg_f32x4{0.f, 0.f, 0.f, 0.f};
+  const gg_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll 2
+  for (int k = 0; k < K; k += 32) {
+    gg_bf16x8 wv[2], av[NT];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) wv[u] = wlive[u] ? *reinterpret_cast<const gg_bf16x8*>(wrow[u] + k) : zero;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) av[t] = item[t] >= 0 ? *reinterpret_cast<const gg_bf16x8*>(arow[t] + k) : zero;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u], av[t], acc[u][t], 0, 0, 0);
+  }
+  // lane holds out[row = t * 16 + col][feature f0 + u * 16 + kq * 4 + i], i = 0..3
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    if (item[t] < 0) continue;
+    const size_t dst = out_scatter ? (size_t)item[t] : (size_t)(tile * TM + t * 16 + col);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int f = f0 + u * 16 + kq * 4;
+      TO* op = out + dst * out_stride + f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float v = act ? gelu_erf(acc[u][t][i]) : acc[u][t][i];
+        if (f + i < n_out) op[i] = from_float<TO>(v);
+      }
+    }
+  }
+}
+
 // out[n, :] = sum_j weights[n, j] * (ids[n, j] < n_experts ? part[n * top + j, :] : h[n, :]) + sigmoid(gate[n]) * shared[n, :]
 template <typename T, typename TS>
 __global__ void __launch_bounds__(256)
@@ -218,22 +296,46 @@ extern "C" int ms_moe_route(const float* logits, long long ld, const float* corr
 
 extern "C" int ms_moe_tile_rows() { return GM; }
 
-extern "C" int ms_moe_align(const int* ids, int n_items, int n_experts, int tiles, int* rows, int* tile_expert,
+// tile: rows of a tile, 16 (the tile of every product here) or 64 (of the matrix-core product alone)
+extern "C" int ms_moe_align(const int* ids, int n_items, int n_experts, int tile, int tiles, int* rows, int* tile_expert,
                             hipStream_t stream) {
   if (n_items <= 0 || tiles <= 0) return MS_OK;
-  if (n_experts <= 0) return MS_BAD_ARG;
+  if (n_experts <= 0 || (tile != GM && tile != 4 * GM)) return MS_BAD_ARG;
   if (n_experts > 4096) return MS_UNSUPPORTED;
-  if ((long long)tiles * GM < (long long)n_items + (long long)n_experts * (GM - 1)) return MS_BAD_ARG;
-  moe_align_kernel<<<1, 1024, (2 * n_experts + 1) * sizeof(int), stream>>>(ids, n_items, n_experts, GM, tiles, rows,
+  if ((long long)tiles * tile < (long long)n_items + (long long)n_experts * (tile - 1)) return MS_BAD_ARG;
+  moe_align_kernel<<<1, 1024, (2 * n_experts + 1) * sizeof(int), stream>>>(ids, n_items, n_experts, tile, tiles, rows,
                                                                           tile_expert);
   return ms_launch_status();
 }
 
+// Whether ms_grouped_gemm takes the product to the matrix cores (tiles of `tile` rows).
+extern "C" int ms_grouped_gemm_mfma_ok(int K, long long in_stride, long long out_stride, int tile, int dtype, int out_dtype) {
+  return dtype == MS_BF16 && K % 32 == 0 && in_stride % 8 == 0 && (tile == GM || tile == 4 * GM) &&
+         (out_dtype == MS_F32 || out_dtype == MS_BF16);
+}
+
 extern "C" int ms_grouped_gemm(const void* in, long long in_stride, const void* w, const int* rows, const int* tile_expert,
-                               void* out, long long out_stride, int tiles, int n_out, int K, int in_div, int out_scatter,
-                               int act, int dtype, int out_dtype, hipStream_t stream) {
+                               void* out, long long out_stride, int tiles, int tile, int n_out, int K, int in_div,
+                               int out_scatter, int act, int dtype, int out_dtype, hipStream_t stream) {
   if (tiles <= 0) return MS_OK;
   if (n_out <= 0 || K <= 0 || in_div < 0) return MS_BAD_ARG;
+  if (ms_grouped_gemm_mfma_ok(K, in_stride, out_stride, tile, dtype, out_dtype) && ((uintptr_t)in % 16) == 0 &&
+      ((uintptr_t)w % 16) == 0) {
+    const int slabs = (n_out + GG_SLAB - 1) / GG_SLAB;
+    if (tiles > 65535) return MS_UNSUPPORTED;
+    dim3 grid(slabs, tiles), block(256);
+#define LAUNCH_M(NT, TO)                                                                                              \
+  grouped_gemm_mfma_kernel<NT, TO><<<grid, block, 0, stream>>>((const bf16*)in, (size_t)in_stride, (const bf16*)w, rows, \
+                                                               tile_expert, (TO*)out, (size_t)out_stride, n_out, K,   \
+                                                               in_div, out_scatter, act)
+    if (tile == GM && out_dtype == MS_F32) LAUNCH_M(1, float);
+    else if (tile == GM) LAUNCH_M(1, bf16);
+    else if (out_dtype == MS_F32) LAUNCH_M(4, float);
+    else LAUNCH_M(4, bf16);
+#undef LAUNCH_M
+    return ms_launch_status();
+  }
+  if (tile != GM) return MS_UNSUPPORTED;
   const int cb = (n_out + GN - 1) / GN;
   if (cb > 65535) return MS_UNSUPPORTED;
   dim3 grid(tiles, cb), block(256);

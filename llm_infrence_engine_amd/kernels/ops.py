@@ -65,10 +65,10 @@ _SIGNATURES = {
                                    _c_ptr, _c_int, _c_ptr],
     "ms_attention_mfma_supported": [_c_int, _c_int],
     "ms_paged_attention_mfma": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll,
-                                _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+                                _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr, _c_ptr],
     "ms_paged_attention_mfma_decode": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                                        _c_ll, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
-                                       _c_int, _c_int, _c_int, _c_ptr],
+                                       _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
     "ms_argmax": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr],
     "ms_sample": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                   _c_ptr],
@@ -102,9 +102,10 @@ _SIGNATURES = {
     "ms_gelu": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_moe_route": [_c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "ms_moe_tile_rows": [],
-    "ms_moe_align": [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
+    "ms_moe_align": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
+    "ms_grouped_gemm_mfma_ok": [_c_int, _c_ll, _c_ll, _c_int, _c_int, _c_int],
     "ms_grouped_gemm": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                        _c_int, _c_int, _c_ptr],
+                        _c_int, _c_int, _c_int, _c_ptr],
     "ms_moe_combine": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_ptr, _c_int, _c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int,
                        _c_int, _c_int, _c_ptr],
 }
@@ -780,13 +781,16 @@ def attention_splits_keys(n_requests: int, num_kv_heads: int, group: int, max_q_
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch.Tensor, block_table: torch.Tensor,
                          q_start: torch.Tensor, context_lens: torch.Tensor, out: torch.Tensor, num_heads: int,
                          scale: float, max_q_len: int, max_context_len: int, window: Optional[int] = None,
-                         table_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+                         table_rows: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Matrix-core attention, bfloat16.  k_pages [P, nkv, page_size, d], vt_pages [P, nkv, d, page_size];
     request r owns tokens q_start[r]..q_start[r+1]-1, holds context_lens[r] keys after this step and has row
     ``table_rows[r]`` of ``block_table`` (row r without ``table_rows``).  ``max_q_len`` and ``max_context_len``
     are upper bounds; tokens from q_start[R] on belong to no request, a request may have no token.  A small
-    batch of single tokens with long contexts also splits the keys over blocks (and combines)."""
+    batch of single tokens with long contexts also splits the keys over blocks (and combines).  ``sink`` float [nh]:
+    exp(sink[h]) joins the denominator of head h's softmax."""
     _check(k_pages, "k_pages", torch.bfloat16)
+    if sink is not None:
+        _check(sink, "sink", torch.float32, (num_heads,))
     P, nkv, page_size, d = k_pages.shape
     _check(vt_pages, "vt_pages", torch.bfloat16, (P, nkv, d, page_size))
     _check(q, "q", torch.bfloat16, contiguous=False)
@@ -823,12 +827,12 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch
         _call("ms_paged_attention_mfma_decode", q.data_ptr(), q_stride, k_pages.data_ptr(), vt_pages.data_ptr(),
               block_table.data_ptr(), block_table.shape[1], _ptr(table_rows), q_start.data_ptr(), context_lens.data_ptr(),
               out.data_ptr(), num_heads * d, part_o.data_ptr(), part_ml.data_ptr(), R, num_heads, nkv, d, page_size, float(scale),
-              int(window or 0), MIN_BLOCKS_PER_SPLIT, n_splits, _stream())
+              int(window or 0), MIN_BLOCKS_PER_SPLIT, n_splits, _ptr(sink), _stream())
     else:
         _call("ms_paged_attention_mfma", q.data_ptr(), q_stride, k_pages.data_ptr(), vt_pages.data_ptr(),
               block_table.data_ptr(), block_table.shape[1], _ptr(table_rows), q_start.data_ptr(), context_lens.data_ptr(),
               out.data_ptr(), num_heads * d, R, N, max_q_len, num_heads, nkv, d, page_size, float(scale), int(window or 0),
-              _stream())
+              _ptr(sink), _stream())
     return out
 
 
@@ -873,7 +877,7 @@ def paged_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, num_heads: int,
     ``sink`` float [num_heads]: exp(sink[h]) joins the denominator of head h's softmax."""
     d, page_size = kv.k_pages.shape[3], kv.k_pages.shape[2]
     dv = kv.v_pages.shape[2] if kv.v_transposed else kv.v_pages.shape[3]
-    if dv != d or sink is not None:
+    if dv != d:
         return paged_attention_generic(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.token_req, ctx.positions, out,
                                        num_heads, scale, window, kv.v_transposed, kv.table_rows, ctx.n_live_tokens, sink)
     if q.dtype == torch.bfloat16 and not (kv.v_transposed and attention_mfma_supported(d, page_size)):
@@ -883,9 +887,9 @@ def paged_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, num_heads: int,
     if (q.dtype == torch.bfloat16 and kv.v_transposed and attention_mfma_supported(d, page_size)
             and q.data_ptr() % 16 == 0 and (q.shape[0] == 1 or q.stride(0) % 8 == 0)):
         return paged_attention_mfma(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.q_start, ctx.context_lens, out,
-                                    num_heads, scale, ctx.max_q_len, ctx.max_context_len, window, kv.table_rows)
+                                    num_heads, scale, ctx.max_q_len, ctx.max_context_len, window, kv.table_rows, sink)
     return paged_attention_generic(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.token_req, ctx.positions, out,
-                                   num_heads, scale, window, kv.v_transposed, kv.table_rows, ctx.n_live_tokens)
+                                   num_heads, scale, window, kv.v_transposed, kv.table_rows, ctx.n_live_tokens, sink)
 
 
 # ------------------------------------------------------------------------------------------------ state-carrying mixers
@@ -1258,18 +1262,25 @@ def moe_tile_rows() -> int:
     return int(_get("ms_moe_tile_rows")())
 
 
-def moe_align(ids: torch.Tensor, n_experts: int):
-    """Groups the rows (token, choice) of ``ids`` [N, top] by expert into tiles of ``moe_tile_rows()`` rows of one expert
-    each.  Returns (rows int32 [tiles * tile]: the flat index n * top + j of every row or -1, tile_expert int32 [tiles]:
-    the tile's expert or -1).  Choices >= n_experts (experts without weights) take no row.  The number of tiles depends
-    on the sizes alone."""
+def moe_wide_tiles_pay(n_items: int, n_experts: int, K: int, dtype: torch.dtype) -> bool:
+    """Whether the grouped products of ``n_items`` rows over ``n_experts`` experts should run in tiles of four times
+    ``moe_tile_rows()`` rows: on the matrix cores (bfloat16, K a multiple of 32), once an expert has some 32 rows on
+    average, a wide tile reads the expert's matrix a quarter as often."""
+    return dtype == torch.bfloat16 and K % 32 == 0 and n_items >= 32 * n_experts
+
+
+def moe_align(ids: torch.Tensor, n_experts: int, wide: bool = False):
+    """Groups the rows (token, choice) of ``ids`` [N, top] by expert into tiles of ``moe_tile_rows()`` rows (``wide``:
+    four times as many) of one expert each.  Returns (rows int32 [tiles * tile]: the flat index n * top + j of every
+    row or -1, tile_expert int32 [tiles]: the tile's expert or -1).  Choices >= n_experts (experts without weights) take
+    no row.  The number of tiles depends on the sizes alone."""
     _check(ids, "ids", torch.int32)
     n_items = ids.numel()
-    tile = moe_tile_rows()
+    tile = moe_tile_rows() * (4 if wide else 1)
     tiles = (n_items + n_experts * (tile - 1) + tile - 1) // tile
     rows = torch.empty(tiles * tile, dtype=torch.int32, device=ids.device)
     tile_expert = torch.empty(tiles, dtype=torch.int32, device=ids.device)
-    _call("ms_moe_align", ids.data_ptr(), n_items, n_experts, tiles, rows.data_ptr(), tile_expert.data_ptr(), _stream())
+    _call("ms_moe_align", ids.data_ptr(), n_items, n_experts, tile, tiles, rows.data_ptr(), tile_expert.data_ptr(), _stream())
     return rows, tile_expert
 
 
@@ -1277,17 +1288,21 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, rows: torch.Tensor, tile_expe
                  gather_div: int = 0, scatter: bool = False, act: Optional[str] = None) -> torch.Tensor:
     """For every tile with an expert e and every row of it (flat position p, item = rows[p] >= 0):
     out[item if scatter else p] = act(a[item // gather_div if gather_div else p] @ w[e].T); w [experts, n_out, K]; float
-    accumulation in the order of K.  ``act``: None or "gelu"."""
+    accumulation in the order of K.  ``act``: None or "gelu".  The tiles' size is read off ``rows`` and ``tile_expert``
+    (``moe_align``'s); bfloat16 with K a multiple of 32 runs on the matrix cores, everything else on the vector ALUs
+    (tiles of ``moe_tile_rows()`` rows only)."""
     _check(w, "w", a.dtype)
     if w.dim() != 3:
         raise ValueError("w must be [experts, out features, in features]")
     E, n_out, K = w.shape
     a_stride = _rows2d(a, "a", None, K)
     o_stride = _rows2d(out, "out", None, n_out)
-    tile = moe_tile_rows()
-    tiles = tile_expert.numel()
-    _check(rows, "rows", torch.int32, (tiles * tile,))
     _check(tile_expert, "tile_expert", torch.int32)
+    tiles = tile_expert.numel()
+    _check(rows, "rows", torch.int32)
+    tile = rows.numel() // max(1, tiles)
+    if tile * tiles != rows.numel() or tile not in (moe_tile_rows(), 4 * moe_tile_rows()):
+        raise ValueError(f"{rows.numel()} rows do not make {tiles} tiles of {moe_tile_rows()} or {4 * moe_tile_rows()}")
     if not gather_div and a.shape[0] < tiles * tile:
         raise ValueError("a must hold a row for every row of every tile")
     if not scatter and out.shape[0] < tiles * tile:
@@ -1295,8 +1310,8 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, rows: torch.Tensor, tile_expe
     if act not in (None, "gelu"):
         raise ValueError(f"no activation {act!r} here")
     _call("ms_grouped_gemm", a.data_ptr(), a_stride, w.data_ptr(), rows.data_ptr(), tile_expert.data_ptr(), out.data_ptr(),
-          o_stride, tiles, n_out, K, int(gather_div), int(scatter), int(act == "gelu"), _code(a.dtype), _code(out.dtype),
-          _stream())
+          o_stride, tiles, tile, n_out, K, int(gather_div), int(scatter), int(act == "gelu"), _code(a.dtype),
+          _code(out.dtype), _stream())
     return out
 
 

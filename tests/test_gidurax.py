@@ -520,6 +520,55 @@ def test_attention_with_a_sink_and_a_loud_far_key(dtype, H, G, D, E, page):
 
 
 @gpu
+@pytest.mark.parametrize("H,G,D", [(8, 2, 64), (4, 4, 32), (14, 2, 128)])
+def test_sink_attention_when_single_tokens_are_decoded(H, G, D):
+    """A step of single tokens in bfloat16 over contexts short and long (beyond the length from which a small batch's
+    keys are split over blocks and combined): the matrix-core kernels with the sink, against the plain attention."""
+    from llm_infrence_engine_amd.kernels import ops
+
+    g = torch.Generator().manual_seed(H + D)
+    page, lens = 16, [1300, 40, 700]
+    sink = torch.tensor([4.0, -3.0, 6.0, 7.0, -1.0, 0.0, 5.5, 3.0, 1.0, 2.0, 8.0, -2.0, 4.5, 6.5][:H])
+    scale, rep = 1.1 / math.sqrt(D), H // G
+    qs, want, tables, kps, vps, base = [], [], [], [], [], 1
+    for T in lens:
+        q = torch.randn(1, H, D, generator=g).bfloat16()
+        k = torch.randn(T, G, D, generator=g).bfloat16()
+        v = torch.randn(T, G, D, generator=g).bfloat16()
+        k[5, 0] = (5.0 * q[0, 0].float() / q[0, 0].float().norm()).bfloat16()          # a loud key near the start
+        full_q = torch.zeros(T, H, D, dtype=torch.float64)
+        full_q[T - 1] = q[0].double()
+        want.append(P.sink_softmax_attention(full_q, k.double().repeat_interleave(rep, 1), v.double().repeat_interleave(rep, 1),
+                                             scale, sink.double())[T - 1])
+        n = -(-T // page)
+        order = [base + int(i) for i in np.random.default_rng(T).permutation(n)]
+        kp, vp, table = _paged(k, v, page, order, torch.bfloat16, True)
+        kps.append(kp), vps.append(vp), tables.append(table[1]), qs.append(q.reshape(1, H * D))
+        base += n
+    P_ = base + 1
+    k_pages = torch.zeros(P_, G, page, D, dtype=torch.bfloat16, device="cuda")
+    v_pages = torch.zeros(P_, G, D, page, dtype=torch.bfloat16, device="cuda")
+    width = max(t.numel() for t in tables)
+    table = torch.zeros(len(lens) + 1, width, dtype=torch.int32, device="cuda")
+    for r, (kp, vp, tb) in enumerate(zip(kps, vps, tables)):
+        used = tb[tb > 0].long()
+        k_pages[used], v_pages[used] = kp[used], vp[used]
+        table[r + 1, :tb.numel()] = tb
+    ctx = _Ctx([1] * len(lens), [0] * len(lens), [T - 1 for T in lens])
+
+    class KV:
+        pass
+
+    kv = KV()
+    kv.k_pages, kv.v_pages, kv.v_transposed, kv.block_table = k_pages, v_pages, True, table
+    kv.table_rows = torch.tensor([1, 2, 3], dtype=torch.int32, device="cuda")
+    out = torch.empty(len(lens), H * D, dtype=torch.bfloat16, device="cuda")
+    ops.paged_attention(torch.cat(qs).cuda(), kv, ctx, out, H, scale, None, sink.cuda())
+    for r in range(len(lens)):
+        assert (out[r].cpu().double().reshape(H, D) - want[r]).abs().max() < 3e-2, r
+
+
+@gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,E,page", [(6, 2, 16, 24, 4), (2, 1, 40, 8, 8), (4, 4, 64, 64, 16)])
 def test_head_norm_temperature_and_cache_store(dtype, H, G, D, E, page):
@@ -559,16 +608,17 @@ def test_head_norm_temperature_and_cache_store(dtype, H, G, D, E, page):
 
 @gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("E,I,top,F_,S_", [(5, 2, 2, 40, 56), (7, 0, 1, 64, 0), (4, 1, 3, 48, 0), (70, 3, 6, 24, 32)])
-def test_routed_experts_alone(dtype, E, I, top, F_, S_):
-    """The part against the plain feed-forward for 37 tokens: choices (identities among them: the correction pushes
-    them in), weights, experts, the shared expert and its gate."""
+@pytest.mark.parametrize("E,I,top,F_,S_,W,N", [(5, 2, 2, 40, 56, 72, 37), (7, 0, 1, 64, 0, 72, 37), (4, 1, 3, 48, 0, 72, 37),
+                                               (70, 3, 6, 24, 32, 72, 37), (6, 2, 3, 96, 0, 64, 40), (4, 1, 2, 64, 32, 96, 300)])
+def test_routed_experts_alone(dtype, E, I, top, F_, S_, W, N):
+    """The part against the plain feed-forward: choices (identities among them: the correction pushes them in),
+    weights, experts, the shared expert and its gate.  The last two shapes run on the matrix cores in bfloat16, in
+    tiles of 16 rows and (300 tokens) of 64."""
     from llm_infrence_engine_amd.kernels import ops
     from llm_infrence_engine_amd.parts.base import Runtime
     from llm_infrence_engine_amd.parts.experts import RoutedExperts
 
     g = torch.Generator().manual_seed(E * 10 + top)
-    W, N = 72, 37
     r = lambda *s: torch.randn(*s, generator=g)
     w = {"m.router": (r(E + I, W) * 0.4).to(dtype), "m.correction": torch.cat([0.05 * r(E), 0.3 + 0.05 * r(I)]).to(dtype)}
     for e in range(E):
@@ -594,14 +644,16 @@ def test_routed_experts_alone(dtype, E, I, top, F_, S_):
     assert torch.equal(ids.cpu().long().sort(1).values, chosen.sort(1).values)
     assert torch.allclose(wts.cpu().double().sort(1).values, weights.sort(1).values, atol=1e-6)
     # the grouping: every (token, choice) of an expert with tensors sits in exactly one row of a tile of its expert
-    rows, tile_expert = ops.moe_align(ids, E)
-    rows, tile_expert, flat = rows.cpu(), tile_expert.cpu(), ids.cpu().reshape(-1)
-    tile = ops.moe_tile_rows()
-    seen = rows[rows >= 0]
-    assert sorted(seen.tolist()) == [i for i in range(N * top) if flat[i] < E]
-    for p_, item in enumerate(rows.tolist()):
-        if item >= 0:
-            assert tile_expert[p_ // tile] == flat[item]
+    flat = ids.cpu().reshape(-1)
+    for wide in (False, True):
+        rows, tile_expert = (t.cpu() for t in ops.moe_align(ids, E, wide))
+        tile = ops.moe_tile_rows() * (4 if wide else 1)
+        assert rows.numel() == tile * tile_expert.numel()
+        seen = rows[rows >= 0]
+        assert sorted(seen.tolist()) == [i for i in range(N * top) if flat[i] < E]
+        for p_, item in enumerate(rows.tolist()):
+            if item >= 0:
+                assert tile_expert[p_ // tile] == flat[item]
 
 
 # ================================================================================================ whole models (GPU)
