@@ -235,8 +235,9 @@ int ms_gelu(const void* x, void* out, long long total, int dtype, hipStream_t st
 int ms_moe_route(const float* logits, long long ld, const float* correction, int n_tokens, int n_out, int top, int* ids,
                  float* weights, hipStream_t stream);
 int ms_moe_tile_rows();
+int ms_moe_wide_tile_rows();
 // rows [tiles * tile] and tile_expert [tiles] from ids [n_items]; ids >= n_experts take no row; tile: ms_moe_tile_rows()
-// or four times that (for the matrix-core product alone)
+// or ms_moe_wide_tile_rows() (for the matrix-core product alone)
 int ms_moe_align(const int* ids, int n_items, int n_experts, int tile, int tiles, int* rows, int* tile_expert,
                  hipStream_t stream);
 int ms_grouped_gemm_mfma_ok(int K, long long in_stride, long long out_stride, int tile, int dtype, int out_dtype);

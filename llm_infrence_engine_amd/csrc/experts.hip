@@ -245,6 +245,107 @@ grouped_gemm_mfma_kernel(const bf16* __restrict__ in, size_t in_stride, const bf
   }
 }
 
+// The product for tiles of 128 rows, for experts with many rows each (portions of prompts).  A block owns a tile and 256
+// output features, 64 to each wave: 32 accumulator tiles a wave, so a row of the expert's matrix that a wave reads serves
+// 128 rows of activations and the activations, which all waves need, are staged once a block through LDS (two buffers
+// taken in turn, one barrier a step of 32 along K).  The next step's rows of the matrix and activations are asked for
+// before the current step's products start.
+constexpr int GW_NT = 8, GW_FT = 4, GW_TM = 16 * GW_NT, GW_SLAB = 64 * 4, GW_KS = 32, GW_PAD = 8;
+
+template <typename TO>
+__global__ void __launch_bounds__(256, 2)
+grouped_gemm_mfma_wide_kernel(const bf16* __restrict__ in, size_t in_stride, const bf16* __restrict__ w,
+                              const int* __restrict__ rows, const int* __restrict__ tile_expert, TO* __restrict__ out,
+                              size_t out_stride, int n_out, int K, int in_div, int out_scatter, int act) {
+  __shared__ __align__(16) bf16 Bs[2][GW_TM][GW_KS + GW_PAD];
+  __shared__ int s_item[GW_TM];
+  const int tile = blockIdx.y;
+  const int e = tile_expert[tile];
+  if (e < 0) return;
+  const int tid = threadIdx.x, lane = tid & (MS_WAVE - 1), wave = tid / MS_WAVE;
+  const int col = lane & 15, kq = lane >> 4;
+  if (tid < GW_TM) s_item[tid] = rows[tile * GW_TM + tid];
+  __syncthreads();
+  // staging: a row of a step is 64 bytes, four pieces of 16; a thread brings two pieces
+  const bf16* src[2];
+  bool src_live[2];
+  int st_row[2], st_part[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int c = tid + j * 256;
+    st_row[j] = c >> 2;
+    st_part[j] = c & 3;
+    const int item = s_item[st_row[j]];
+    src_live[j] = item >= 0;
+    const size_t r = in_div > 0 ? (size_t)(max(item, 0) / in_div) : (size_t)(tile * GW_TM + st_row[j]);
+    src[j] = in + r * in_stride + st_part[j] * 8;
+  }
+  const int f0 = blockIdx.x * GW_SLAB + wave * 64;
+  const bf16* we = w + (size_t)e * n_out * K;
+  const bf16* wrow[GW_FT];
+  bool wlive[GW_FT];
+#pragma unroll
+  for (int u = 0; u < GW_FT; ++u) {
+    const int f = f0 + u * 16 + col;
+    wlive[u] = f < n_out;
+    wrow[u] = we + (size_t)(wlive[u] ? f : 0) * K + kq * 8;
+  }
+  gg_f32x4 acc[GW_FT][GW_NT];
+#pragma unroll
+  for (int u = 0; u < GW_FT; ++u)
+#pragma unroll
+    for (int t = 0; t < GW_NT; ++t) acc[u][t] = gg_f32x4{0.f, 0.f, 0.f, 0.f};
+  const gg_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  gg_bf16x8 gb[2], wv[GW_FT], wn[GW_FT];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) gb[j] = src_live[j] ? *reinterpret_cast<const gg_bf16x8*>(src[j]) : zero;
+#pragma unroll
+  for (int u = 0; u < GW_FT; ++u) wv[u] = wlive[u] ? *reinterpret_cast<const gg_bf16x8*>(wrow[u]) : zero;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) *reinterpret_cast<gg_bf16x8*>(&Bs[0][st_row[j]][st_part[j] * 8]) = gb[j];
+  __syncthreads();
+  int cur = 0;
+  for (int k = 0; k < K; k += GW_KS) {
+    const bool more = k + GW_KS < K;
+    if (more) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) gb[j] = src_live[j] ? *reinterpret_cast<const gg_bf16x8*>(src[j] + k + GW_KS) : zero;
+#pragma unroll
+      for (int u = 0; u < GW_FT; ++u) wn[u] = wlive[u] ? *reinterpret_cast<const gg_bf16x8*>(wrow[u] + k + GW_KS) : zero;
+    }
+#pragma unroll
+    for (int t = 0; t < GW_NT; ++t) {
+      const gg_bf16x8 bv = *reinterpret_cast<const gg_bf16x8*>(&Bs[cur][t * 16 + col][kq * 8]);
+#pragma unroll
+      for (int u = 0; u < GW_FT; ++u) acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u], bv, acc[u][t], 0, 0, 0);
+    }
+    if (more) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) *reinterpret_cast<gg_bf16x8*>(&Bs[cur ^ 1][st_row[j]][st_part[j] * 8]) = gb[j];
+#pragma unroll
+      for (int u = 0; u < GW_FT; ++u) wv[u] = wn[u];
+    }
+    __syncthreads();
+    cur ^= 1;
+  }
+#pragma unroll
+  for (int t = 0; t < GW_NT; ++t) {
+    const int item = s_item[t * 16 + col];
+    if (item < 0) continue;
+    const size_t dst = out_scatter ? (size_t)item : (size_t)(tile * GW_TM + t * 16 + col);
+#pragma unroll
+    for (int u = 0; u < GW_FT; ++u) {
+      const int f = f0 + u * 16 + kq * 4;
+      TO* op = out + dst * out_stride + f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float v = act ? gelu_erf(acc[u][t][i]) : acc[u][t][i];
+        if (f + i < n_out) op[i] = from_float<TO>(v);
+      }
+    }
+  }
+}
+
 // out[n, :] = sum_j weights[n, j] * (ids[n, j] < n_experts ? part[n * top + j, :] : h[n, :]) + sigmoid(gate[n]) * shared[n, :]
 template <typename T, typename TS>
 __global__ void __launch_bounds__(256)
@@ -295,12 +396,13 @@ extern "C" int ms_moe_route(const float* logits, long long ld, const float* corr
 }
 
 extern "C" int ms_moe_tile_rows() { return GM; }
+extern "C" int ms_moe_wide_tile_rows() { return GW_TM; }
 
-// tile: rows of a tile, 16 (the tile of every product here) or 64 (of the matrix-core product alone)
+// tile: rows of a tile, 16 (the tile of every product here) or 128 (of the matrix-core product alone)
 extern "C" int ms_moe_align(const int* ids, int n_items, int n_experts, int tile, int tiles, int* rows, int* tile_expert,
                             hipStream_t stream) {
   if (n_items <= 0 || tiles <= 0) return MS_OK;
-  if (n_experts <= 0 || (tile != GM && tile != 4 * GM)) return MS_BAD_ARG;
+  if (n_experts <= 0 || (tile != GM && tile != GW_TM)) return MS_BAD_ARG;
   if (n_experts > 4096) return MS_UNSUPPORTED;
   if ((long long)tiles * tile < (long long)n_items + (long long)n_experts * (tile - 1)) return MS_BAD_ARG;
   moe_align_kernel<<<1, 1024, (2 * n_experts + 1) * sizeof(int), stream>>>(ids, n_items, n_experts, tile, tiles, rows,
@@ -310,7 +412,7 @@ extern "C" int ms_moe_align(const int* ids, int n_items, int n_experts, int tile
 
 // Whether ms_grouped_gemm takes the product to the matrix cores (tiles of `tile` rows).
 extern "C" int ms_grouped_gemm_mfma_ok(int K, long long in_stride, long long out_stride, int tile, int dtype, int out_dtype) {
-  return dtype == MS_BF16 && K % 32 == 0 && in_stride % 8 == 0 && (tile == GM || tile == 4 * GM) &&
+  return dtype == MS_BF16 && K % 32 == 0 && in_stride % 8 == 0 && (tile == GM || tile == GW_TM) &&
          (out_dtype == MS_F32 || out_dtype == MS_BF16);
 }
 
@@ -321,18 +423,24 @@ extern "C" int ms_grouped_gemm(const void* in, long long in_stride, const void* 
   if (n_out <= 0 || K <= 0 || in_div < 0) return MS_BAD_ARG;
   if (ms_grouped_gemm_mfma_ok(K, in_stride, out_stride, tile, dtype, out_dtype) && ((uintptr_t)in % 16) == 0 &&
       ((uintptr_t)w % 16) == 0) {
-    const int slabs = (n_out + GG_SLAB - 1) / GG_SLAB;
+    const int slab = tile == GM ? GG_SLAB : GW_SLAB;
+    const int slabs = (n_out + slab - 1) / slab;
     if (tiles > 65535) return MS_UNSUPPORTED;
     dim3 grid(slabs, tiles), block(256);
+#define LAUNCH_W(TO)                                                                                                  \
+  grouped_gemm_mfma_wide_kernel<TO><<<grid, block, 0, stream>>>((const bf16*)in, (size_t)in_stride, (const bf16*)w, rows, \
+                                                                tile_expert, (TO*)out, (size_t)out_stride, n_out, K,  \
+                                                                in_div, out_scatter, act)
 #define LAUNCH_M(NT, TO)                                                                                              \
   grouped_gemm_mfma_kernel<NT, TO><<<grid, block, 0, stream>>>((const bf16*)in, (size_t)in_stride, (const bf16*)w, rows, \
                                                                tile_expert, (TO*)out, (size_t)out_stride, n_out, K,   \
                                                                in_div, out_scatter, act)
     if (tile == GM && out_dtype == MS_F32) LAUNCH_M(1, float);
     else if (tile == GM) LAUNCH_M(1, bf16);
-    else if (out_dtype == MS_F32) LAUNCH_M(4, float);
-    else LAUNCH_M(4, bf16);
+    else if (out_dtype == MS_F32) LAUNCH_W(float);
+    else LAUNCH_W(bf16);
 #undef LAUNCH_M
+#undef LAUNCH_W
     return ms_launch_status();
   }
   if (tile != GM) return MS_UNSUPPORTED;

@@ -56,7 +56,7 @@ selective_scan_kernel(const T* __restrict__ x, size_t x_stride, const float* __r
     const int n = part * SPT + i;
     const bool in = live && n < states;
     S[i] = in ? Sg[n] : 0.f;
-    a[i] = in ? A[(size_t)ch * states + n] : 0.f;
+    a[i] = in ? A[(size_t)ch * states + n] * 1.4426950408889634f : 0.f;   // exp(dt a) = 2^(dt a log2 e)
   }
   const float dskip = live ? Dskip[ch] : 0.f;
   for (int t0 = 0; t0 < L; t0 += SCAN_CHUNK) {
@@ -78,21 +78,38 @@ selective_scan_kernel(const T* __restrict__ x, size_t x_stride, const float* __r
       s_c[t][i] = i < states ? to_float(C[n * bc_stride + i]) : 0.f;
     }
     __syncthreads();
-    for (int t = 0; t < cn; ++t) {
+    // one token: everything but the last multiply-add of a state is independent of the state, so the tokens of a
+    // group of four overlap; the exponential is the hardware's 2^x
+    auto token = [&](int t) __attribute__((always_inline)) -> float {
       const float dt = s_dt[t][ch_local], xv = s_x[t][ch_local];
       const float dx = dt * xv;
       float acc = 0.f;
 #pragma unroll
       for (int i = 0; i < SPT; ++i) {
-        S[i] = fmaf(expf(dt * a[i]), S[i], dx * s_b[t][part * SPT + i]);
+        S[i] = fmaf(__builtin_amdgcn_exp2f(dt * a[i]), S[i], dx * s_b[t][part * SPT + i]);
         acc = fmaf(S[i], s_c[t][part * SPT + i], acc);
       }
-      acc = scan_group_sum<LPC>(acc);
-      if (live && part == 0) {
-        const float zv = s_z[t][ch_local];
-        const float y = fmaf(dskip, xv, acc);
-        out[(size_t)(s0 + t0 + t) * out_stride + ch] = from_float<T>(y * (zv / (1.0f + expf(-zv))));
+      return fmaf(dskip, xv, scan_group_sum<LPC>(acc));
+    };
+    auto gate_store = [&](int t, float y) __attribute__((always_inline)) {
+      const float zv = s_z[t][ch_local];
+      const float g = sizeof(T) == 4 ? zv / (1.0f + expf(-zv)) : fast_silu(zv);
+      out[(size_t)(s0 + t0 + t) * out_stride + ch] = from_float<T>(y * g);
+    };
+    int t = 0;
+    if (LPC >= 4) {
+      // four tokens at a time; then lane u of a channel's group gates and stores token u, so that the gate's
+      // arithmetic runs once for the four tokens and not once for each
+      for (; t + 4 <= cn; t += 4) {
+        const float y0 = token(t), y1 = token(t + 1), y2 = token(t + 2), y3 = token(t + 3);
+        const int u = part & 3;
+        const float y = u == 0 ? y0 : (u == 1 ? y1 : (u == 2 ? y2 : y3));
+        if (live && part < 4) gate_store(t + u, y);
       }
+    }
+    for (; t < cn; ++t) {
+      const float y = token(t);
+      if (live && part == 0) gate_store(t, y);
     }
   }
 #pragma unroll

@@ -102,6 +102,7 @@ _SIGNATURES = {
     "ms_gelu": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_moe_route": [_c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "ms_moe_tile_rows": [],
+    "ms_moe_wide_tile_rows": [],
     "ms_moe_align": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "ms_grouped_gemm_mfma_ok": [_c_int, _c_ll, _c_ll, _c_int, _c_int, _c_int],
     "ms_grouped_gemm": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -1262,21 +1263,25 @@ def moe_tile_rows() -> int:
     return int(_get("ms_moe_tile_rows")())
 
 
+def moe_wide_tile_rows() -> int:
+    return int(_get("ms_moe_wide_tile_rows")())
+
+
 def moe_wide_tiles_pay(n_items: int, n_experts: int, K: int, dtype: torch.dtype) -> bool:
-    """Whether the grouped products of ``n_items`` rows over ``n_experts`` experts should run in tiles of four times
-    ``moe_tile_rows()`` rows: on the matrix cores (bfloat16, K a multiple of 32), once an expert has some 32 rows on
-    average, a wide tile reads the expert's matrix a quarter as often."""
-    return dtype == torch.bfloat16 and K % 32 == 0 and n_items >= 32 * n_experts
+    """Whether the grouped products of ``n_items`` rows over ``n_experts`` experts should run in tiles of
+    ``moe_wide_tile_rows()`` rows: on the matrix cores (bfloat16, K a multiple of 32), once an expert has a wide tile's
+    rows on average, so that most tiles are full; a wide tile reads the expert's matrix an eighth as often."""
+    return dtype == torch.bfloat16 and K % 32 == 0 and n_items >= moe_wide_tile_rows() * n_experts
 
 
 def moe_align(ids: torch.Tensor, n_experts: int, wide: bool = False):
     """Groups the rows (token, choice) of ``ids`` [N, top] by expert into tiles of ``moe_tile_rows()`` rows (``wide``:
-    four times as many) of one expert each.  Returns (rows int32 [tiles * tile]: the flat index n * top + j of every
+    of ``moe_wide_tile_rows()``) of one expert each.  Returns (rows int32 [tiles * tile]: the flat index n * top + j of every
     row or -1, tile_expert int32 [tiles]: the tile's expert or -1).  Choices >= n_experts (experts without weights) take
     no row.  The number of tiles depends on the sizes alone."""
     _check(ids, "ids", torch.int32)
     n_items = ids.numel()
-    tile = moe_tile_rows() * (4 if wide else 1)
+    tile = moe_wide_tile_rows() if wide else moe_tile_rows()
     tiles = (n_items + n_experts * (tile - 1) + tile - 1) // tile
     rows = torch.empty(tiles * tile, dtype=torch.int32, device=ids.device)
     tile_expert = torch.empty(tiles, dtype=torch.int32, device=ids.device)
@@ -1301,8 +1306,8 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, rows: torch.Tensor, tile_expe
     tiles = tile_expert.numel()
     _check(rows, "rows", torch.int32)
     tile = rows.numel() // max(1, tiles)
-    if tile * tiles != rows.numel() or tile not in (moe_tile_rows(), 4 * moe_tile_rows()):
-        raise ValueError(f"{rows.numel()} rows do not make {tiles} tiles of {moe_tile_rows()} or {4 * moe_tile_rows()}")
+    if tile * tiles != rows.numel() or tile not in (moe_tile_rows(), moe_wide_tile_rows()):
+        raise ValueError(f"{rows.numel()} rows do not make {tiles} tiles of {moe_tile_rows()} or {moe_wide_tile_rows()}")
     if not gather_div and a.shape[0] < tiles * tile:
         raise ValueError("a must hold a row for every row of every tile")
     if not scatter and out.shape[0] < tiles * tile:

@@ -48,7 +48,7 @@ class RoutedExperts(FeedForward):
         self.w_up = torch.stack([t[f"e{e}.up"] for e in range(self.experts)]).contiguous()       # [E, F, W]
         self.w_down = torch.stack([t[f"e{e}.down"] for e in range(self.experts)]).contiguous()   # [E, W, F]
         # the router and the shared expert's gate read the same h: one product, float out
-        self.w_router = torch.cat([t["router"]] + ([t["shared.sg"]] if self.shared_ff else []), dim=0).contiguous()
+        self.w_router = linear.prepare_weight(torch.cat([t["router"]] + ([t["shared.sg"]] if self.shared_ff else []), dim=0))
         self.correction = t["correction"]
         if self.shared_ff:
             self.w_shared_up, self.w_shared_down = linear.prepare_weight(t["shared.up"]), linear.prepare_weight(t["shared.down"])
@@ -56,7 +56,7 @@ class RoutedExperts(FeedForward):
     def forward(self, h, ctx):
         N, W, E = h.shape[0], self.hidden_size, self.experts
         n_out = E + self.identity
-        logits = ops.gemm_generic(h, self.w_router, torch.empty((N, self.w_router.shape[0]), dtype=torch.float32, device=h.device))
+        logits = linear.linear(h, self.w_router, out_dtype=torch.float32)
         ids, weights = ops.moe_route(logits, self.correction, self.top, n_out)
         wide = ops.moe_wide_tiles_pay(ids.numel(), E, min(W, self.expert_ff), h.dtype) and W % 32 == 0 and self.expert_ff % 32 == 0
         rows, tile_expert = ops.moe_align(ids, E, wide)

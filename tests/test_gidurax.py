@@ -609,11 +609,11 @@ def test_head_norm_temperature_and_cache_store(dtype, H, G, D, E, page):
 @gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("E,I,top,F_,S_,W,N", [(5, 2, 2, 40, 56, 72, 37), (7, 0, 1, 64, 0, 72, 37), (4, 1, 3, 48, 0, 72, 37),
-                                               (70, 3, 6, 24, 32, 72, 37), (6, 2, 3, 96, 0, 64, 40), (4, 1, 2, 64, 32, 96, 300)])
+                                               (70, 3, 6, 24, 32, 72, 37), (6, 2, 3, 96, 0, 64, 40), (4, 1, 2, 64, 32, 96, 300), (3, 0, 2, 288, 0, 160, 400)])
 def test_routed_experts_alone(dtype, E, I, top, F_, S_, W, N):
     """The part against the plain feed-forward: choices (identities among them: the correction pushes them in),
     weights, experts, the shared expert and its gate.  The last two shapes run on the matrix cores in bfloat16, in
-    tiles of 16 rows and (300 tokens) of 64."""
+    tiles of 16 rows and (the last two) of 128; the very last has more features than a block's slab."""
     from llm_infrence_engine_amd.kernels import ops
     from llm_infrence_engine_amd.parts.base import Runtime
     from llm_infrence_engine_amd.parts.experts import RoutedExperts
@@ -637,7 +637,7 @@ def test_routed_experts_alone(dtype, E, I, top, F_, S_, W, N):
     part.load(lambda s: (w[s.name].float() if s.role != "matrix" else w[s.name].to(dtype)).cuda(), Runtime(torch.device("cuda"), dtype))
     got = part.forward(h.cuda(), None)
     assert got.dtype == torch.float32
-    assert (got.cpu().double() - want).abs().max() < (2e-5 if dtype == torch.float32 else 6e-2)
+    assert (got.cpu().double() - want).abs().max() < (2e-5 if dtype == torch.float32 else 6e-2) * max(1.0, float(want.abs().max()) / 4)
     # the router alone: the same choices (as sets) and the same weights
     logits = (h.double() @ w64["m.router"].T).float().cuda()
     ids, wts = ops.moe_route(logits, w["m.correction"].float().cuda(), top)
@@ -647,7 +647,7 @@ def test_routed_experts_alone(dtype, E, I, top, F_, S_, W, N):
     flat = ids.cpu().reshape(-1)
     for wide in (False, True):
         rows, tile_expert = (t.cpu() for t in ops.moe_align(ids, E, wide))
-        tile = ops.moe_tile_rows() * (4 if wide else 1)
+        tile = ops.moe_wide_tile_rows() if wide else ops.moe_tile_rows()
         assert rows.numel() == tile * tile_expert.numel()
         seen = rows[rows >= 0]
         assert sorted(seen.tolist()) == [i for i in range(N * top) if flat[i] < E]
