@@ -248,9 +248,10 @@ grouped_gemm_mfma_kernel(const bf16* __restrict__ in, size_t in_stride, const bf
 // The product for tiles of 128 rows, for experts with many rows each (portions of prompts).  A block owns a tile and 256
 // output features, 64 to each wave: 32 accumulator tiles a wave, so a row of the expert's matrix that a wave reads serves
 // 128 rows of activations and the activations, which all waves need, are staged once a block through LDS (two buffers
-// taken in turn, one barrier a step of 32 along K).  The next step's rows of the matrix and activations are asked for
+// taken in turn, one barrier a step of 64 along K).  The next step's rows of the matrix and activations are asked for
 // before the current step's products start.
-constexpr int GW_NT = 8, GW_FT = 4, GW_TM = 16 * GW_NT, GW_SLAB = 64 * 4, GW_KS = 32, GW_PAD = 8;
+constexpr int GW_NT = 8, GW_FT = 4, GW_TM = 16 * GW_NT, GW_SLAB = 64 * 4, GW_KS = 64, GW_PAD = 8;
+constexpr int GW_PIECES = GW_TM * (GW_KS / 8) / 256;     // pieces of 16 bytes a thread stages a step
 
 template <typename TO>
 __global__ void __launch_bounds__(256, 2)
@@ -261,20 +262,20 @@ grouped_gemm_mfma_wide_kernel(const bf16* __restrict__ in, size_t in_stride, con
   __shared__ int s_item[GW_TM];
   const int tile = blockIdx.y;
   const int e = tile_expert[tile];
-  if (e < 0) return;
+  if (e < 0 || (int)blockIdx.x * GW_SLAB >= n_out) return;   // an unused tile, or a slab that only pads the grid
   const int tid = threadIdx.x, lane = tid & (MS_WAVE - 1), wave = tid / MS_WAVE;
   const int col = lane & 15, kq = lane >> 4;
   if (tid < GW_TM) s_item[tid] = rows[tile * GW_TM + tid];
   __syncthreads();
-  // staging: a row of a step is 64 bytes, four pieces of 16; a thread brings two pieces
-  const bf16* src[2];
-  bool src_live[2];
-  int st_row[2], st_part[2];
+  // staging: a row of a step is 128 bytes, eight pieces of 16; a thread brings four pieces
+  const bf16* src[GW_PIECES];
+  bool src_live[GW_PIECES];
+  int st_row[GW_PIECES], st_part[GW_PIECES];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < GW_PIECES; ++j) {
     const int c = tid + j * 256;
-    st_row[j] = c >> 2;
-    st_part[j] = c & 3;
+    st_row[j] = c / (GW_KS / 8);
+    st_part[j] = c % (GW_KS / 8);
     const int item = s_item[st_row[j]];
     src_live[j] = item >= 0;
     const size_t r = in_div > 0 ? (size_t)(max(item, 0) / in_div) : (size_t)(tile * GW_TM + st_row[j]);
@@ -296,34 +297,43 @@ grouped_gemm_mfma_wide_kernel(const bf16* __restrict__ in, size_t in_stride, con
 #pragma unroll
     for (int t = 0; t < GW_NT; ++t) acc[u][t] = gg_f32x4{0.f, 0.f, 0.f, 0.f};
   const gg_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  gg_bf16x8 gb[2], wv[GW_FT], wn[GW_FT];
+  gg_bf16x8 gb[GW_PIECES], wv[2][GW_FT], wn[2][GW_FT];
+  // K is a multiple of 32: the last step may hold one half only
+  auto ask = [&](int k, gg_bf16x8 (&wa)[2][GW_FT]) __attribute__((always_inline)) {
 #pragma unroll
-  for (int j = 0; j < 2; ++j) gb[j] = src_live[j] ? *reinterpret_cast<const gg_bf16x8*>(src[j]) : zero;
+    for (int j = 0; j < GW_PIECES; ++j)
+      gb[j] = (src_live[j] && k + st_part[j] * 8 < K) ? *reinterpret_cast<const gg_bf16x8*>(src[j] + k) : zero;
 #pragma unroll
-  for (int u = 0; u < GW_FT; ++u) wv[u] = wlive[u] ? *reinterpret_cast<const gg_bf16x8*>(wrow[u]) : zero;
+    for (int h = 0; h < 2; ++h)
 #pragma unroll
-  for (int j = 0; j < 2; ++j) *reinterpret_cast<gg_bf16x8*>(&Bs[0][st_row[j]][st_part[j] * 8]) = gb[j];
+      for (int u = 0; u < GW_FT; ++u)
+        wa[h][u] = (wlive[u] && k + h * 32 < K) ? *reinterpret_cast<const gg_bf16x8*>(wrow[u] + k + h * 32) : zero;
+  };
+  auto put = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < GW_PIECES; ++j) *reinterpret_cast<gg_bf16x8*>(&Bs[buf][st_row[j]][st_part[j] * 8]) = gb[j];
+  };
+  ask(0, wv);
+  put(0);
   __syncthreads();
   int cur = 0;
   for (int k = 0; k < K; k += GW_KS) {
     const bool more = k + GW_KS < K;
+    if (more) ask(k + GW_KS, wn);
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int t = 0; t < GW_NT; ++t) {
+        const gg_bf16x8 bv = *reinterpret_cast<const gg_bf16x8*>(&Bs[cur][t * 16 + col][h * 32 + kq * 8]);
+#pragma unroll
+        for (int u = 0; u < GW_FT; ++u) acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[h][u], bv, acc[u][t], 0, 0, 0);
+      }
     if (more) {
+      put(cur ^ 1);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) gb[j] = src_live[j] ? *reinterpret_cast<const gg_bf16x8*>(src[j] + k + GW_KS) : zero;
+      for (int h = 0; h < 2; ++h)
 #pragma unroll
-      for (int u = 0; u < GW_FT; ++u) wn[u] = wlive[u] ? *reinterpret_cast<const gg_bf16x8*>(wrow[u] + k + GW_KS) : zero;
-    }
-#pragma unroll
-    for (int t = 0; t < GW_NT; ++t) {
-      const gg_bf16x8 bv = *reinterpret_cast<const gg_bf16x8*>(&Bs[cur][t * 16 + col][kq * 8]);
-#pragma unroll
-      for (int u = 0; u < GW_FT; ++u) acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u], bv, acc[u][t], 0, 0, 0);
-    }
-    if (more) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) *reinterpret_cast<gg_bf16x8*>(&Bs[cur ^ 1][st_row[j]][st_part[j] * 8]) = gb[j];
-#pragma unroll
-      for (int u = 0; u < GW_FT; ++u) wv[u] = wn[u];
+        for (int u = 0; u < GW_FT; ++u) wv[h][u] = wn[h][u];
     }
     __syncthreads();
     cur ^= 1;
