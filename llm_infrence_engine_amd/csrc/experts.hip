@@ -17,8 +17,17 @@ __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + e
 
 template <typename T>
 __global__ void gelu_kernel(const T* __restrict__ x, T* __restrict__ out, size_t total) {
+  constexpr int V = 16 / sizeof(T);     // values in 16 bytes
+  struct alignas(16) Pack { T v[V]; };
   const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride)
+  const size_t packs = (((size_t)x | (size_t)out) & 15) == 0 ? total / V : 0;   // 16 bytes a lane where both are aligned
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < packs; i += stride) {
+    Pack p = reinterpret_cast<const Pack*>(x)[i];
+#pragma unroll
+    for (int j = 0; j < V; ++j) p.v[j] = from_float<T>(gelu_erf(to_float(p.v[j])));
+    reinterpret_cast<Pack*>(out)[i] = p;
+  }
+  for (size_t i = packs * V + (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride)
     out[i] = from_float<T>(gelu_erf(to_float(x[i])));
 }
 
@@ -215,7 +224,8 @@ grouped_gemm_mfma_kernel(const bf16* __restrict__ in, size_t in_stride, const bf
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[u][t] = gg_f32x4{0.f, 0.f, 0.f, 0.f};
   const gg_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll 2
+  // a decode step is the stream of the chosen experts' matrices: four steps' loads in flight a wave
+#pragma unroll 4
   for (int k = 0; k < K; k += 32) {
     gg_bf16x8 wv[2], av[NT];
 #pragma unroll
@@ -387,7 +397,7 @@ moe_combine_kernel(const float* __restrict__ part, const int* __restrict__ ids, 
 
 extern "C" int ms_gelu(const void* x, void* out, long long total, int dtype, hipStream_t stream) {
   if (total <= 0) return MS_OK;
-  int blocks = (int)((total + 1023) / 1024);
+  int blocks = (int)((total / 4 + 255) / 256) + 1;
   if (blocks > 8192) blocks = 8192;
   if (dtype == MS_F32) gelu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)x, (float*)out, (size_t)total);
   else if (dtype == MS_BF16) gelu_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)x, (bf16*)out, (size_t)total);

@@ -5,7 +5,7 @@
 // S float [slots, channels, states] is carried from step to step in the request's slot.  A row of S (one channel) is
 // held in the registers of LPC neighbouring lanes, SPT states each, for the whole portion.  Tokens are staged a chunk
 // at a time: all threads of the block work out the chunk's step sizes (bias, softplus) and convert its x, z, B and C
-// into LDS, then every thread walks the chunk's tokens in order.  Step sizes, exponentials and the state are float.
+// into LDS (asked for a chunk ahead), then every thread walks the chunk's tokens in order.  Step sizes, exponentials and the state are float.
 // A step is a ragged batch: request r owns the tokens q_start[r] .. q_start[r+1]-1 and the slot state_slots[r];
 // requests without tokens are left alone.
 #include "common.h"
@@ -59,25 +59,67 @@ selective_scan_kernel(const T* __restrict__ x, size_t x_stride, const float* __r
     a[i] = in ? A[(size_t)ch * states + n] * 1.4426950408889634f : 0.f;   // exp(dt a) = 2^(dt a log2 e)
   }
   const float dskip = live ? Dskip[ch] : 0.f;
+  // Staging.  A thread asks for its share of the next chunk (raw values, into registers) before it walks the current
+  // one, so that a chunk's trip to memory is over by the time the chunk before has been walked.
+  constexpr int EPT = (SCAN_CHUNK * CPB + SCAN_THREADS - 1) / SCAN_THREADS;   // (token, channel) pairs a thread stages
+  constexpr int BPT = (SCAN_CHUNK * NP + SCAN_THREADS - 1) / SCAN_THREADS;    // (token, state) pairs
+  float dt_r[EPT];
+  T x_r[EPT], z_r[EPT], b_r[BPT], c_r[BPT];
+  auto ask = [&](int t0) __attribute__((always_inline)) {
+    const int cn = min(SCAN_CHUNK, L - t0);
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      const int e = tid + j * SCAN_THREADS;
+      const int t = e / CPB, cl = e - t * CPB;
+      const int c = c0 + cl;
+      if (t < cn && c < channels) {
+        const size_t n = (size_t)(s0 + t0 + t);
+        dt_r[j] = dt_in[n * channels + c] + dt_bias[c];
+        x_r[j] = x[n * x_stride + c];
+        z_r[j] = z[n * z_stride + c];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < BPT; ++j) {
+      const int e = tid + j * SCAN_THREADS;
+      const int t = e / NP, i = e - t * NP;
+      if (t < cn && i < states) {
+        const size_t n = (size_t)(s0 + t0 + t);
+        b_r[j] = B[n * bc_stride + i];
+        c_r[j] = C[n * bc_stride + i];
+      }
+    }
+  };
+  auto stage = [&](int t0) __attribute__((always_inline)) {
+    const int cn = min(SCAN_CHUNK, L - t0);
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      const int e = tid + j * SCAN_THREADS;
+      const int t = e / CPB, cl = e - t * CPB;
+      if (t < cn) {
+        const bool in = c0 + cl < channels;
+        s_dt[t][cl] = in ? scan_softplus(dt_r[j]) : 0.f;
+        s_x[t][cl] = in ? to_float(x_r[j]) : 0.f;
+        s_z[t][cl] = in ? to_float(z_r[j]) : 0.f;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < BPT; ++j) {
+      const int e = tid + j * SCAN_THREADS;
+      const int t = e / NP, i = e - t * NP;
+      if (t < cn) {
+        s_b[t][i] = i < states ? to_float(b_r[j]) : 0.f;
+        s_c[t][i] = i < states ? to_float(c_r[j]) : 0.f;
+      }
+    }
+  };
+  ask(0);
   for (int t0 = 0; t0 < L; t0 += SCAN_CHUNK) {
     const int cn = min(SCAN_CHUNK, L - t0);
     __syncthreads();    // the chunk before has been walked
-    for (int e = tid; e < cn * CPB; e += SCAN_THREADS) {
-      const int t = e / CPB, cl = e - t * CPB;
-      const int c = c0 + cl;
-      const size_t n = (size_t)(s0 + t0 + t);
-      const bool in = c < channels;
-      s_dt[t][cl] = in ? scan_softplus(dt_in[n * channels + c] + dt_bias[c]) : 0.f;
-      s_x[t][cl] = in ? to_float(x[n * x_stride + c]) : 0.f;
-      s_z[t][cl] = in ? to_float(z[n * z_stride + c]) : 0.f;
-    }
-    for (int e = tid; e < cn * NP; e += SCAN_THREADS) {
-      const int t = e / NP, i = e - t * NP;
-      const size_t n = (size_t)(s0 + t0 + t);
-      s_b[t][i] = i < states ? to_float(B[n * bc_stride + i]) : 0.f;
-      s_c[t][i] = i < states ? to_float(C[n * bc_stride + i]) : 0.f;
-    }
+    stage(t0);
     __syncthreads();
+    if (t0 + SCAN_CHUNK < L) ask(t0 + SCAN_CHUNK);
     // one token: everything but the last multiply-add of a state is independent of the state, so the tokens of a
     // group of four overlap; the exponential is the hardware's 2^x
     auto token = [&](int t) __attribute__((always_inline)) -> float {
