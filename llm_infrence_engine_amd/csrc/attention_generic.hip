@@ -1,5 +1,4 @@
-// Paged causal attention with grouped heads, any key size that is a multiple of 4 up to 256 and any value size up
-// to 256, for any mix of prompt portions and single decoded tokens.  `sink` (may be null): one number per query
+// Paged causal attention with grouped heads, any key size and any value size up to 256, for any mix of prompt portions and single decoded tokens.  `sink` (may be null): one number per query
 // head whose exponential joins the softmax's denominator; it has no key and no value.  One wave per (token, query head): scores, running
 // maximum, exponentials, their sum and the weighted sum of values are all float.  It reads keys and
 // values in place through the request's block table and never reads a key beyond the token's own
@@ -59,12 +58,14 @@ paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T
       row = (page * nkv + kvh) * page_size + (j % page_size);
       const T* kp = k_pages + (size_t)row * d;
       float dot = 0.f;
-      for (int i = 0; i < d; i += 4) {
+      int i = 0;
+      for (; i + 3 < d; i += 4) {
         dot = fmaf(qs[wave][i], to_float(kp[i]), dot);
         dot = fmaf(qs[wave][i + 1], to_float(kp[i + 1]), dot);
         dot = fmaf(qs[wave][i + 2], to_float(kp[i + 2]), dot);
         dot = fmaf(qs[wave][i + 3], to_float(kp[i + 3]), dot);
       }
+      for (; i < d; ++i) dot = fmaf(qs[wave][i], to_float(kp[i]), dot);
       s = dot;
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -111,7 +112,7 @@ extern "C" int ms_paged_attention_generic(const void* q, long long q_stride, con
   if (n_tokens <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || page_size <= 0 || table_stride <= 0)
     return MS_BAD_ARG;
-  if (head_dim <= 0 || head_dim % 4 || head_dim > MAX_D || value_dim <= 0 || value_dim > MAX_D) return MS_UNSUPPORTED;
+  if (head_dim <= 0 || head_dim > MAX_D || value_dim <= 0 || value_dim > MAX_D) return MS_UNSUPPORTED;
   if (num_pages * num_kv_heads * page_size >= (1ll << 31)) return MS_UNSUPPORTED;  // row index is an int
   const long long items = (long long)n_tokens * num_heads;
   dim3 grid((unsigned)((items + WAVES - 1) / WAVES)), block(WAVES * MS_WAVE);

@@ -29,8 +29,8 @@ class GQAttention(Mixer):
                  value_dim: Optional[int] = None, sink: bool = False, names=None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads cannot share {num_kv_heads} key/value heads")
-        if head_dim % 4 or head_dim > 256:
-            raise ValueError(f"head_dim {head_dim} is not supported: the attention kernels take multiples of 4 up to 256")
+        if not 0 < head_dim <= 256:
+            raise ValueError(f"head_dim {head_dim} is not supported: the attention kernels take sizes up to 256")
         if window is not None and window <= 0:
             raise ValueError("window must be positive")
         self.prefix, self.position = prefix, position

@@ -480,7 +480,7 @@ def _paged(keys, vals, page, order, dtype, transposed=False):
 
 @gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,D,E,page", [(6, 2, 16, 24, 4), (4, 1, 64, 64, 16), (3, 3, 32, 8, 8), (8, 2, 64, 64, 16)])
+@pytest.mark.parametrize("H,G,D,E,page", [(6, 2, 16, 24, 4), (4, 1, 64, 64, 16), (3, 3, 32, 8, 8), (8, 2, 64, 64, 16), (2, 1, 6, 10, 4)])
 def test_attention_with_a_sink_and_a_loud_far_key(dtype, H, G, D, E, page):
     """One sequence of 300 tokens in pages in no order: the last 40 queries attend over everything.  One key far back
     (at a page's last slot) is made loud for one query, so that leaving it out, or being one token off, shows; sinks of

@@ -456,10 +456,10 @@ def test_ops_refuse_cpu_tensors_and_wrong_shapes(ops):
     with pytest.raises(ValueError):
         ops.silu_mul(torch.zeros(2, 4, device=DEV), torch.zeros(2, 3, device=DEV))
     with pytest.raises(RuntimeError, match="unsupported"):
-        kp = torch.zeros(2, 1, 4, 6, device=DEV)  # head size 6 is no multiple of 4
-        ops.paged_attention_generic(torch.zeros(1, 6, device=DEV), kp, kp, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+        kp = torch.zeros(2, 1, 4, 260, device=DEV)  # head sizes go up to 256
+        ops.paged_attention_generic(torch.zeros(1, 260, device=DEV), kp, kp, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
                                     torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
-                                    torch.zeros(1, 6, device=DEV), 1, 1.0)
+                                    torch.zeros(1, 260, device=DEV), 1, 1.0)
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
