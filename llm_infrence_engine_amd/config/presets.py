@@ -51,7 +51,7 @@ def _gidurax(width, ff, layers, scan, delta, attention, experts, vocab=151936):
     ef, n, ident, top, shared = experts
     routed = {"kind": "moe", "expert": {"ff": ef}, "router": {"experts": n, "identity": ident, "top": top}, "shared": {"ff": shared}}
     kinds = [("mamba1", scan), ("delta", delta), ("attention", attention), ("attention", attention)]
-    return {"architecture": "Gidurax", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.7,
+    return {"architecture": "Gidurax", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
             "embedding": {"scale": float(width) ** 0.5},
             "layers": [{"type": kinds[i % 4][0], "mixer": dict(kinds[i % 4][1]),
                         "mlp": dict(routed) if i % 2 else {"kind": "dense", "ff": ff}} for i in range(layers)]}
@@ -62,12 +62,12 @@ def _gidurax(width, ff, layers, scan, delta, attention, experts, vocab=151936):
 PRESETS["gidurax-0.5b"] = _gidurax(
     896, 7296, 24, {"inner": 1792, "state": 16, "dt_rank": 56, "conv": 4},
     {"heads": 14, "kv_heads": 7, "dim": 64, "vdim": 64, "conv": 4},
-    {"heads": 14, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.125, "q_temp": {"coef": 0.3, "every": 128}},
+    {"heads": 14, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 64 ** -0.5, "q_temp": {"coef": 0.25, "every": 256}},
     (1824, 16, 2, 3, 1824))
 PRESETS["gidurax-7b"] = _gidurax(
     3584, 28416, 28, {"inner": 7168, "state": 16, "dt_rank": 224, "conv": 4},
     {"heads": 28, "kv_heads": 14, "dim": 128, "vdim": 128, "conv": 4},
-    {"heads": 28, "kv_heads": 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "q_temp": {"coef": 0.3, "every": 128}},
+    {"heads": 28, "kv_heads": 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "q_temp": {"coef": 0.25, "every": 256}},
     (7104, 16, 2, 3, 7104), vocab=152064)
 
 

@@ -72,11 +72,15 @@ SHAPES = {
         mamba_layer(40, 130, 3, 4, None)]),
 }
 # heads of 64 with pages of 16: in bfloat16 this attention runs on the matrix cores
-SHAPES["S"] = config(257, 160, 1e-5, 0.7, 12.6, [
-    attention_layer(8, 2, 64, 64, 0.125, moe(64, 6, 2, identity=1, shared=64), temp=(0.3, 32)),
+SHAPES["S"] = config(257, 160, 1e-5, 0.75, 12.6, [
+    attention_layer(6, 2, 64, 64, 0.11, moe(64, 6, 2, identity=1, shared=64), temp=(0.35, 32)),
     mamba_layer(192, 16, 6, 4, dense(192)),
     attention_layer(4, 4, 32, 32, 0.18, dense(128))], loop=(0, 1, 2))
 PAGES = {"P": 16, "Q": 8, "R": 4, "S": 16}
+# seeds of the shapes' weights.  A router's choice is a comparison of floats: with some weights a token's last chosen and
+# first unchosen expert lie closer together than bfloat16 activations can tell apart, and the two precisions then run
+# different experts for that token, which no bound on rounding covers; these seeds have no such token in the tests' requests
+SEEDS = {"P": ord("P"), "Q": ord("Q"), "R": ord("R"), "S": 1001}
 
 
 def tensor_shapes(cfg):
@@ -480,7 +484,8 @@ def _paged(keys, vals, page, order, dtype, transposed=False):
 
 @gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,D,E,page", [(6, 2, 16, 24, 4), (4, 1, 64, 64, 16), (3, 3, 32, 8, 8), (8, 2, 64, 64, 16), (2, 1, 6, 10, 4)])
+@pytest.mark.parametrize("H,G,D,E,page", [(6, 2, 16, 24, 4), (4, 1, 64, 64, 16), (3, 3, 32, 8, 8), (8, 2, 64, 64, 16), (2, 1, 6, 10, 4),
+                                          (6, 2, 64, 64, 16), (3, 1, 128, 128, 16), (5, 1, 32, 32, 16)])
 def test_attention_with_a_sink_and_a_loud_far_key(dtype, H, G, D, E, page):
     """One sequence of 300 tokens in pages in no order: the last 40 queries attend over everything.  One key far back
     (at a page's last slot) is made loud for one query, so that leaving it out, or being one token off, shows; sinks of
@@ -609,11 +614,13 @@ def test_head_norm_temperature_and_cache_store(dtype, H, G, D, E, page):
 @gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("E,I,top,F_,S_,W,N", [(5, 2, 2, 40, 56, 72, 37), (7, 0, 1, 64, 0, 72, 37), (4, 1, 3, 48, 0, 72, 37),
-                                               (70, 3, 6, 24, 32, 72, 37), (6, 2, 3, 96, 0, 64, 40), (4, 1, 2, 64, 32, 96, 300), (3, 0, 2, 288, 0, 160, 400)])
+                                               (70, 3, 6, 24, 32, 72, 37), (6, 2, 3, 96, 0, 64, 40), (4, 1, 2, 64, 32, 96, 300), (3, 0, 2, 288, 0, 160, 400),
+                                               (4, 1, 2, 192, 0, 128, 300), (3, 0, 2, 320, 64, 256, 400)])
 def test_routed_experts_alone(dtype, E, I, top, F_, S_, W, N):
     """The part against the plain feed-forward: choices (identities among them: the correction pushes them in),
     weights, experts, the shared expert and its gate.  The last two shapes run on the matrix cores in bfloat16, in
-    tiles of 16 rows and (the last two) of 128; the very last has more features than a block's slab."""
+    tiles of 16 rows and (the last four) of 128: two on the kernel that reads its operands in place or through registers,
+    two (sizes that are multiples of 64) on the tiled kernel, with fewer and more features than a block's tile."""
     from llm_infrence_engine_amd.kernels import ops
     from llm_infrence_engine_amd.parts.base import Runtime
     from llm_infrence_engine_amd.parts.experts import RoutedExperts
@@ -672,7 +679,7 @@ def rounded_forward(cfg, w, toks):
 def shape(request, tmp_path_factory):
     name = request.param
     cfg = SHAPES[name]
-    weights = random_weights(cfg, seed=ord(name))
+    weights = random_weights(cfg, seed=SEEDS[name])
     folder = write_model(tmp_path_factory.mktemp("gidurax" + name), cfg, weights)
     lengths = {"P": [5, 61, 2, 130, 33, 48], "Q": [1, 9, 90, 47, 110, 64], "R": [3, 26, 70, 17, 2, 41, 60, 33],
                "S": [70, 3, 140, 50, 97, 33]}[name]
@@ -809,7 +816,7 @@ def test_greedy_generation_through_the_engine(shape, dtype):
     import llm_infrence_engine_amd as eng
 
     name, cfg, folder, reqs, want, noise = shape
-    weights = {k: v.double() for k, v in random_weights(cfg, seed=ord(name)).items()}
+    weights = {k: v.double() for k, v in random_weights(cfg, seed=SEEDS[name]).items()}
     prompts = [toks[:max(1, len(toks) // 3)] for toks in list(reqs.values())[:4]]
     llm = eng.LLM(str(folder), dtype=dtype, block_size=PAGES[name], max_len=128, max_seqs=3, max_prefill_chunk=7)
     outs = llm.generate(prompts, eng.SamplingParams(max_new_tokens=12))
