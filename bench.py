@@ -80,6 +80,10 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
     rng = np.random.default_rng(seed)
     budget = max(4096, batch)
     extra = -(-batch * prompt_len // budget) + 2     # requests admitted first decode while the others prefill
+    # graphs that draw tokens are captured at first use; the timed steps end with a launch of steps % (steps a launch)
+    # steps, whose graph the warm-up must have used too
+    tail = steps % DECODE_STEPS_PER_LAUNCH if sampling else 0
+    extra += tail
     need = prompt_len + warmup + steps + extra
     pages = batch * (-(-need // BLOCK_SIZE) + 1)
     e = eng_mod.Engine(model, num_blocks=pages, block_size=BLOCK_SIZE, max_seqs=batch, max_len=CONTEXT_LIMIT,
@@ -100,6 +104,8 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
         assert done == n and all(rec.decode_batch == batch and rec.n_prefill_tokens == 0 for rec in e.steps[first:])
 
     run(warmup)
+    if tail:
+        run(tail)
     assert len(e.running) == batch and all(r.num_tokens - r.num_computed == 1 for r in e.running)
     graphs = e.runner.graphs
     held = len(graphs.buckets)      # (graphs that draw tokens are captured at their first use: the warm-up steps)
@@ -112,7 +118,7 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
     if len(graphs.buckets) != held:
         raise AssertionError("a graph was captured inside the timed region")
     dt = total / steps
-    mean_context = prompt_len + warmup + (steps + 1) / 2
+    mean_context = prompt_len + warmup + tail + (steps + 1) / 2
     launches = graphs.launches - n0
     # the host's share: filling the static buffers and enqueuing the graph, against the whole launch
     launch = {"steps_per_launch": round(steps / launches, 2),
