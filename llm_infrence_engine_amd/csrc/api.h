@@ -237,9 +237,16 @@ int ms_moe_route(const float* logits, long long ld, const float* correction, int
 int ms_moe_tile_rows();
 int ms_moe_wide_tile_rows();
 // rows [tiles * tile] and tile_expert [tiles] from ids [n_items]; ids >= n_experts take no row; tile: ms_moe_tile_rows()
-// or ms_moe_wide_tile_rows() (for the matrix-core product alone)
+// or, for the matrix-core products alone, ms_moe_wide_tile_rows() or ms_gemm_tiled_grouped_rows()
 int ms_moe_align(const int* ids, int n_items, int n_experts, int tile, int tiles, int* rows, int* tile_expert,
                  hipStream_t stream);
+// the same product for tiles of ms_gemm_tiled_grouped_rows() rows, or half as many, on the tiled kernel
+// (csrc/gemm_tiled.hip): K a multiple of 64
+int ms_gemm_tiled_grouped_rows();
+int ms_gemm_tiled_grouped(const void* A, long long lda, const void* W, const int* rows, const int* tile_expert, void* out,
+                          long long ldo, int tiles, int tile_rows, int N, int K, int in_div, int out_scatter, int act,
+                          int out_dtype, hipStream_t stream);
+
 int ms_grouped_gemm_mfma_ok(int K, long long in_stride, long long out_stride, int tile, int dtype, int out_dtype);
 // for every tile t with an expert e and each of its rows i (flat position p = t * tile + i, item = rows[p] >= 0):
 // out[out_scatter ? item : p] = act(w[e] . in[in_div ? item / in_div : p]); w [experts, n_out, K]

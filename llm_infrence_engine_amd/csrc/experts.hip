@@ -418,11 +418,11 @@ extern "C" int ms_moe_route(const float* logits, long long ld, const float* corr
 extern "C" int ms_moe_tile_rows() { return GM; }
 extern "C" int ms_moe_wide_tile_rows() { return GW_TM; }
 
-// tile: rows of a tile, 16 (the tile of every product here) or 128 (of the matrix-core product alone)
+// tile: rows of a tile, 16 (the tile of every product here), or 128 or 256 (of the matrix-core products alone)
 extern "C" int ms_moe_align(const int* ids, int n_items, int n_experts, int tile, int tiles, int* rows, int* tile_expert,
                             hipStream_t stream) {
   if (n_items <= 0 || tiles <= 0) return MS_OK;
-  if (n_experts <= 0 || (tile != GM && tile != GW_TM)) return MS_BAD_ARG;
+  if (n_experts <= 0 || (tile != GM && tile != GW_TM && tile != ms_gemm_tiled_grouped_rows())) return MS_BAD_ARG;
   if (n_experts > 4096) return MS_UNSUPPORTED;
   if ((long long)tiles * tile < (long long)n_items + (long long)n_experts * (tile - 1)) return MS_BAD_ARG;
   moe_align_kernel<<<1, 1024, (2 * n_experts + 1) * sizeof(int), stream>>>(ids, n_items, n_experts, tile, tiles, rows,
@@ -441,6 +441,13 @@ extern "C" int ms_grouped_gemm(const void* in, long long in_stride, const void* 
                                int out_scatter, int act, int dtype, int out_dtype, hipStream_t stream) {
   if (tiles <= 0) return MS_OK;
   if (n_out <= 0 || K <= 0 || in_div < 0) return MS_BAD_ARG;
+  if (tile == ms_gemm_tiled_grouped_rows() || (tile * 2 == ms_gemm_tiled_grouped_rows() && K % 64 == 0 && dtype == MS_BF16)) {
+    // wide tiles with K a multiple of 64: the tiled kernel, operands from memory straight to LDS
+    const int rc = dtype == MS_BF16 ? ms_gemm_tiled_grouped(in, in_stride, w, rows, tile_expert, out, out_stride, tiles,
+                                                            tile, n_out, K, in_div, out_scatter, act, out_dtype, stream)
+                                    : MS_UNSUPPORTED;
+    if (rc != MS_UNSUPPORTED || tile == ms_gemm_tiled_grouped_rows()) return rc;
+  }
   if (ms_grouped_gemm_mfma_ok(K, in_stride, out_stride, tile, dtype, out_dtype) && ((uintptr_t)in % 16) == 0 &&
       ((uintptr_t)w % 16) == 0) {
     const int slab = tile == GM ? GG_SLAB : GW_SLAB;

@@ -23,7 +23,21 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_QKV = 2 };
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_QKV = 2, EPI_GROUPED = 3 };
+
+// What the grouped product needs beside the operands: the token tiles are tiles of rows that belong to one expert each
+// (ms_moe_align's lists), W holds the experts' matrices one after the other, rows of A are gathered and rows of the
+// result scattered by the rows' list.
+struct GroupedRows {
+  const int* rows;          // [m_tiles * BM]: item of every row, < 0: none
+  const int* tile_expert;   // [m_tiles]: the tile's expert, < 0: nobody's tile
+  size_t expert_stride;     // elements between two experts' matrices
+  int in_div;               // > 0: row p of the product reads A[item / in_div]; 0: A[p]
+  int out_scatter;          // the result of row p goes to out[item] (else out[p])
+  int act;                  // 1: the exact gelu of the product
+};
+
+__device__ __forceinline__ float tiled_gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f)); }
 
 // What the q/k/v epilogue needs beside the product: W's rows are [q heads | k heads | v heads] of FT * 16 features.
 struct QkvEpilogue {
@@ -83,11 +97,21 @@ __device__ __forceinline__ void store_run(bf16* o, const float* v, int valid) {
   }
 }
 
+__device__ __forceinline__ void store_run_f32(float* o, const float* v, int run, int valid) {
+  if (valid >= run && run % 4 == 0 && ((uintptr_t)o % 16) == 0) {
+    for (int g = 0; g < run; g += 4) *reinterpret_cast<f32x4*>(o + g) = f32x4{v[g], v[g + 1], v[g + 2], v[g + 3]};
+  } else {
+    for (int g = 0; g < run; ++g)
+      if (g < valid) o[g] = v[g];
+  }
+}
+
 // WF x WT waves along features and tokens, each with FT x TT tiles of 16 x 16.  K is a multiple of 64.
 template <int WF, int WT, int FT, int TT, int EPI, typename TO>
 __global__ void __launch_bounds__(WF * WT * MS_WAVE)
 gemm_tiled_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict__ W, size_t ldw,
-                  TO* __restrict__ out, size_t ldo, int M, int N, int K, int m_tiles, int n_tiles, int xm, QkvEpilogue qkv) {
+                  TO* __restrict__ out, size_t ldo, int M, int N, int K, int m_tiles, int n_tiles, int xm, QkvEpilogue qkv,
+                  GroupedRows grp) {
   constexpr int NWAVES = WF * WT, THREADS = NWAVES * MS_WAVE;
   constexpr int BN = WF * FT * 16, BM = WT * TT * 16, ROWS = BN + BM;
   constexpr int LOADS = (ROWS / 8 + NWAVES - 1) / NWAVES;   // loads of 8 rows (1 KB) a wave makes per step at most
@@ -107,6 +131,11 @@ gemm_tiled_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict
   const int mt = (local % mi) * xm + xcd % xm;
   if (nt >= n_tiles || mt >= m_tiles) return;
   const int n0 = nt * BN, m0 = mt * BM;
+  if (EPI == EPI_GROUPED) {     // the token tile is a tile of one expert's rows: its matrix is the W of this block
+    const int e = grp.tile_expert[mt];
+    if (e < 0) return;
+    W += (size_t)e * grp.expert_stride;
+  }
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int wf = wave % WF, wt = wave / WF;
   const int col = lane & 15, kq = lane >> 4;
@@ -120,7 +149,11 @@ gemm_tiled_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict
     const int l = min((wave + p * NWAVES) * 8 + (lane >> 3), ROWS - 1);   // (past the tile's rows: not loaded)
     const int piece = (lane & 7) ^ (l & 7);
     if (l < BN) src[p] = W + (size_t)min(n0 + feature_of_row<FT>(l), N - 1) * ldw + piece * 8;
-    else src[p] = A + (size_t)min(m0 + l - BN, M - 1) * lda + piece * 8;
+    else {
+      int r = min(m0 + l - BN, M - 1);
+      if (EPI == EPI_GROUPED && grp.in_div > 0) r = max(grp.rows[r], 0) / grp.in_div;   // (a row without an item: any row)
+      src[p] = A + (size_t)r * lda + piece * 8;
+    }
   }
   typedef __attribute__((address_space(3))) void lds_void;
   typedef const __attribute__((address_space(1))) void global_void;
@@ -264,6 +297,15 @@ gemm_tiled_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict
         v[2 * i + 1] = fast_silu(acc[i][j][2]) * acc[i][j][3];
       }
       store_run<2 * FT>(reinterpret_cast<bf16*>(out) + (size_t)m * ldo + o0, v, n_out - o0);
+    } else if (EPI == EPI_GROUPED) {
+      const int item = grp.rows[m];
+      if (item < 0) continue;
+      const size_t row = grp.out_scatter ? (size_t)item : (size_t)m;
+      float v[4 * FT];
+#pragma unroll
+      for (int g = 0; g < 4 * FT; ++g) v[g] = grp.act ? tiled_gelu_erf(acc[g >> 2][j][g & 3]) : acc[g >> 2][j][g & 3];
+      if (sizeof(TO) == 4) store_run_f32(reinterpret_cast<float*>(out) + row * ldo + f0, v, 4 * FT, N - f0);
+      else store_run<4 * FT>(reinterpret_cast<bf16*>(out) + row * ldo + f0, v, N - f0);
     } else {
       float v[4 * FT];
 #pragma unroll
@@ -301,7 +343,32 @@ int launch(const bf16* A, size_t lda, const bf16* W, size_t ldw, TO* out, size_t
   const long long blocks = 8LL * ((m_tiles + xm - 1) / xm) * ((n_tiles + 8 / xm - 1) / (8 / xm));
   if (blocks > 0x7fffffffLL) return MS_UNSUPPORTED;
   gemm_tiled_kernel<WF, WT, FT, TT, EPI, TO><<<dim3((unsigned)blocks), dim3(WF * WT * MS_WAVE), lds, stream>>>(
-      A, lda, W, ldw, out, ldo, M, N, K, m_tiles, n_tiles, xm, qkv);
+      A, lda, W, ldw, out, ldo, M, N, K, m_tiles, n_tiles, xm, qkv, GroupedRows{});
+  return ms_launch_status();
+}
+
+// The grouped product: tiles of 256 features by 256 rows (TT = 4) or 128 rows (TT = 2), the rows' tiles those of
+// ms_moe_align.  The XCDs are laid over the tiles of W alone (xm = 1), row tiles running fastest on an XCD:
+// neighbouring row tiles mostly belong to one expert and then share its slab of W in that XCD's L2 at the same time.
+constexpr int GROUPED_TT = 4;
+template <typename TO, int TT>
+int launch_grouped(const bf16* A, size_t lda, const bf16* W, TO* out, size_t ldo, int tiles, int N, int K,
+                   const GroupedRows& grp, hipStream_t stream) {
+  constexpr int WF = 2, WT = 4, FT = 8;
+  constexpr int BN = WF * FT * 16, BM = WT * TT * 16;
+  constexpr size_t lds = 2 * (size_t)(BN + BM) * PITCH * sizeof(bf16);
+  static bool raised = false;
+  if (!raised) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiled_kernel<WF, WT, FT, TT, EPI_GROUPED, TO>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return MS_LAUNCH_FAILED;
+    raised = true;
+  }
+  const int n_tiles = (N + BN - 1) / BN;
+  const long long blocks = 8LL * tiles * ((n_tiles + 7) / 8);
+  if (blocks > 0x7fffffffLL) return MS_UNSUPPORTED;
+  gemm_tiled_kernel<WF, WT, FT, TT, EPI_GROUPED, TO><<<dim3((unsigned)blocks), dim3(WF * WT * MS_WAVE), lds, stream>>>(
+      A, lda, W, (size_t)K, out, ldo, tiles * BM, N, K, tiles, n_tiles, 1, QkvEpilogue{}, grp);
   return ms_launch_status();
 }
 
@@ -376,6 +443,29 @@ extern "C" int ms_gemm_tiled(const void* A, long long lda, const void* W, long l
   if (tile == 4) GO(2, 4, 6, 4);   // 192 features x 256 tokens
   if (tile == 5) GO(2, 4, 5, 4);   // 160 features x 256 tokens
   GO(2, 4, 4, 2);                  // 128 x 128
+#undef GO
+}
+
+// The grouped product of routed experts on this kernel: for every tile t of tile_rows rows (ms_gemm_tiled_grouped_rows()
+// or half of that) with an expert e and each of its rows p (item = rows[p] >= 0): out[out_scatter ? item : p] =
+// act(W[e] . A[in_div ? item / in_div : p]); W [experts, N, K] bfloat16 with K a multiple of 64, out bfloat16 or float.
+// MS_UNSUPPORTED for what it does not take.
+extern "C" int ms_gemm_tiled_grouped_rows() { return 4 * GROUPED_TT * 16; }
+extern "C" int ms_gemm_tiled_grouped(const void* A, long long lda, const void* W, const int* rows, const int* tile_expert,
+                                     void* out, long long ldo, int tiles, int tile_rows, int N, int K, int in_div,
+                                     int out_scatter, int act, int out_dtype, hipStream_t stream) {
+  if (tiles <= 0 || N <= 0) return MS_OK;
+  if (K <= 0 || K % BK || lda % 8 || lda < K || ldo < N || in_div < 0) return MS_UNSUPPORTED;
+  if (((uintptr_t)A | (uintptr_t)W) % 16) return MS_UNSUPPORTED;
+  const bool whole = tile_rows == ms_gemm_tiled_grouped_rows();
+  if (!whole && tile_rows * 2 != ms_gemm_tiled_grouped_rows()) return MS_UNSUPPORTED;
+  if (out_dtype != MS_BF16 && out_dtype != MS_F32) return MS_BAD_ARG;
+  const GroupedRows grp{rows, tile_expert, (size_t)N * (size_t)K, in_div, out_scatter, act};
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+#define GO(TO, TT) return launch_grouped<TO, TT>(a, (size_t)lda, w, (TO*)out, (size_t)ldo, tiles, N, K, grp, stream)
+  if (out_dtype == MS_BF16) { if (whole) GO(bf16, GROUPED_TT); else GO(bf16, GROUPED_TT / 2); }
+  if (whole) GO(float, GROUPED_TT); else GO(float, GROUPED_TT / 2);
 #undef GO
 }
 

@@ -103,6 +103,7 @@ _SIGNATURES = {
     "ms_moe_route": [_c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "ms_moe_tile_rows": [],
     "ms_moe_wide_tile_rows": [],
+    "ms_gemm_tiled_grouped_rows": [],
     "ms_moe_align": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "ms_grouped_gemm_mfma_ok": [_c_int, _c_ll, _c_ll, _c_int, _c_int, _c_int],
     "ms_grouped_gemm": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -1267,21 +1268,36 @@ def moe_wide_tile_rows() -> int:
     return int(_get("ms_moe_wide_tile_rows")())
 
 
-def moe_wide_tiles_pay(n_items: int, n_experts: int, K: int, dtype: torch.dtype) -> bool:
-    """Whether the grouped products of ``n_items`` rows over ``n_experts`` experts should run in tiles of
-    ``moe_wide_tile_rows()`` rows: on the matrix cores (bfloat16, K a multiple of 32), once an expert has a wide tile's
-    rows on average, so that most tiles are full; a wide tile reads the expert's matrix an eighth as often."""
-    return dtype == torch.bfloat16 and K % 32 == 0 and n_items >= moe_wide_tile_rows() * n_experts
+def moe_widest_tile_rows() -> int:
+    return int(_get("ms_gemm_tiled_grouped_rows")())
 
 
-def moe_align(ids: torch.Tensor, n_experts: int, wide: bool = False):
-    """Groups the rows (token, choice) of ``ids`` [N, top] by expert into tiles of ``moe_tile_rows()`` rows (``wide``:
-    of ``moe_wide_tile_rows()``) of one expert each.  Returns (rows int32 [tiles * tile]: the flat index n * top + j of every
+def moe_tile_choice(n_items: int, n_experts: int, sizes, dtype: torch.dtype) -> int:
+    """The rows of a tile for the grouped products of ``n_items`` rows over ``n_experts`` experts whose matrices have
+    the row lengths ``sizes``.  An expert's matrix is read once for every tile of its rows, so wider tiles read less:
+    on the matrix cores (bfloat16), once an expert has a wide tile's rows on average (so that most tiles are full),
+    ``moe_widest_tile_rows()`` where every size is a multiple of 64 (half-empty tiles cost matrix-core time that the
+    product, bound by the bytes it moves, has to spare), else
+    ``moe_wide_tile_rows()`` where every size is a multiple of 32; ``moe_tile_rows()`` otherwise (a decode step: the
+    chosen experts' matrices stream once)."""
+    if dtype == torch.bfloat16 and n_items >= moe_wide_tile_rows() * n_experts:
+        if all(k % 64 == 0 for k in sizes):
+            return moe_widest_tile_rows()
+        if all(k % 32 == 0 for k in sizes):
+            return moe_wide_tile_rows()
+    return moe_tile_rows()
+
+
+def moe_align(ids: torch.Tensor, n_experts: int, tile: Optional[int] = None):
+    """Groups the rows (token, choice) of ``ids`` [N, top] by expert into tiles of ``tile`` rows (``moe_tile_rows()``,
+    the default, ``moe_wide_tile_rows()`` or ``moe_widest_tile_rows()``) of one expert each.  Returns (rows int32 [tiles * tile]: the flat index n * top + j of every
     row or -1, tile_expert int32 [tiles]: the tile's expert or -1).  Choices >= n_experts (experts without weights) take
     no row.  The number of tiles depends on the sizes alone."""
     _check(ids, "ids", torch.int32)
     n_items = ids.numel()
-    tile = moe_wide_tile_rows() if wide else moe_tile_rows()
+    tile = moe_tile_rows() if tile is None else int(tile)
+    if tile not in (moe_tile_rows(), moe_wide_tile_rows(), moe_widest_tile_rows()):
+        raise ValueError(f"tiles have {moe_tile_rows()}, {moe_wide_tile_rows()} or {moe_widest_tile_rows()} rows, not {tile}")
     tiles = (n_items + n_experts * (tile - 1) + tile - 1) // tile
     rows = torch.empty(tiles * tile, dtype=torch.int32, device=ids.device)
     tile_expert = torch.empty(tiles, dtype=torch.int32, device=ids.device)
@@ -1294,8 +1310,8 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, rows: torch.Tensor, tile_expe
     """For every tile with an expert e and every row of it (flat position p, item = rows[p] >= 0):
     out[item if scatter else p] = act(a[item // gather_div if gather_div else p] @ w[e].T); w [experts, n_out, K]; float
     accumulation in the order of K.  ``act``: None or "gelu".  The tiles' size is read off ``rows`` and ``tile_expert``
-    (``moe_align``'s); bfloat16 with K a multiple of 32 runs on the matrix cores, everything else on the vector ALUs
-    (tiles of ``moe_tile_rows()`` rows only)."""
+    (``moe_align``'s); bfloat16 with K a multiple of 32 runs on the matrix cores (the widest tiles: a multiple of 64),
+    everything else on the vector ALUs (tiles of ``moe_tile_rows()`` rows only)."""
     _check(w, "w", a.dtype)
     if w.dim() != 3:
         raise ValueError("w must be [experts, out features, in features]")
@@ -1306,8 +1322,9 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, rows: torch.Tensor, tile_expe
     tiles = tile_expert.numel()
     _check(rows, "rows", torch.int32)
     tile = rows.numel() // max(1, tiles)
-    if tile * tiles != rows.numel() or tile not in (moe_tile_rows(), moe_wide_tile_rows()):
-        raise ValueError(f"{rows.numel()} rows do not make {tiles} tiles of {moe_tile_rows()} or {moe_wide_tile_rows()}")
+    if tile * tiles != rows.numel() or tile not in (moe_tile_rows(), moe_wide_tile_rows(), moe_widest_tile_rows()):
+        raise ValueError(f"{rows.numel()} rows do not make {tiles} tiles of {moe_tile_rows()}, {moe_wide_tile_rows()} or "
+                         f"{moe_widest_tile_rows()}")
     if not gather_div and a.shape[0] < tiles * tile:
         raise ValueError("a must hold a row for every row of every tile")
     if not scatter and out.shape[0] < tiles * tile:

@@ -58,8 +58,7 @@ class RoutedExperts(FeedForward):
         n_out = E + self.identity
         logits = linear.linear(h, self.w_router, out_dtype=torch.float32)
         ids, weights = ops.moe_route(logits, self.correction, self.top, n_out)
-        wide = ops.moe_wide_tiles_pay(ids.numel(), E, min(W, self.expert_ff), h.dtype) and W % 32 == 0 and self.expert_ff % 32 == 0
-        rows, tile_expert = ops.moe_align(ids, E, wide)
+        rows, tile_expert = ops.moe_align(ids, E, ops.moe_tile_choice(ids.numel(), E, (W, self.expert_ff), h.dtype))
         mid = ops.grouped_gemm(h, self.w_up, rows, tile_expert, self.rt.empty(rows.numel(), self.expert_ff),
                                gather_div=self.top, act=self.activation)
         part = ops.grouped_gemm(mid, self.w_down, rows, tile_expert,

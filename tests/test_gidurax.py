@@ -619,8 +619,8 @@ def test_head_norm_temperature_and_cache_store(dtype, H, G, D, E, page):
 def test_routed_experts_alone(dtype, E, I, top, F_, S_, W, N):
     """The part against the plain feed-forward: choices (identities among them: the correction pushes them in),
     weights, experts, the shared expert and its gate.  The last two shapes run on the matrix cores in bfloat16, in
-    tiles of 16 rows and (the last four) of 128: two on the kernel that reads its operands in place or through registers,
-    two (sizes that are multiples of 64) on the tiled kernel, with fewer and more features than a block's tile."""
+    tiles of 16 rows, (the next two) of 128 and (the last two, whose sizes are multiples of 64) of 256 on the tiled
+    kernel, with fewer and more features than a block's tile."""
     from llm_infrence_engine_amd.kernels import ops
     from llm_infrence_engine_amd.parts.base import Runtime
     from llm_infrence_engine_amd.parts.experts import RoutedExperts
@@ -652,9 +652,8 @@ def test_routed_experts_alone(dtype, E, I, top, F_, S_, W, N):
     assert torch.allclose(wts.cpu().double().sort(1).values, weights.sort(1).values, atol=1e-6)
     # the grouping: every (token, choice) of an expert with tensors sits in exactly one row of a tile of its expert
     flat = ids.cpu().reshape(-1)
-    for wide in (False, True):
-        rows, tile_expert = (t.cpu() for t in ops.moe_align(ids, E, wide))
-        tile = ops.moe_wide_tile_rows() if wide else ops.moe_tile_rows()
+    for tile in (ops.moe_tile_rows(), ops.moe_wide_tile_rows(), ops.moe_widest_tile_rows()):
+        rows, tile_expert = (t.cpu() for t in ops.moe_align(ids, E, tile))
         assert rows.numel() == tile * tile_expert.numel()
         seen = rows[rows >= 0]
         assert sorted(seen.tolist()) == [i for i in range(N * top) if flat[i] < E]
